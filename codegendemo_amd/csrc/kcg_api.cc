@@ -1,0 +1,571 @@
+// kcg_api.cc — the C ABI of libkcg_gemm.so (declared in include/kcg_gemm.h).
+//
+//   compile : config -> instantiation stub -> hiprtc (gfx950) -> code object file, with an on-disk
+//             cache keyed by a hash of everything that determines the binary
+//   load    : code object file -> hipModule / hipFunction
+//   launch  : hipModuleLaunchKernel with three device pointers and dynamic LDS
+//   bench   : HIP-event timing loop in C
+//
+// There is no CPU execution path here: without a HIP device, load/launch/benchmark fail with
+// KCG_ERR_HIP.  Compilation alone needs no device.
+#include <dlfcn.h>
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+#include <sys/types.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "kcg_config.h"
+
+#define KCG_VERSION "kcg-gemm-gfx950 0.1"
+
+// The device template header, embedded at build time (path given by -DKCG_DEVICE_HEADER_PATH).
+__asm__(
+    ".section .rodata\n"
+    ".global kcg_device_src\n"
+    "kcg_device_src:\n"
+    ".incbin \"" KCG_DEVICE_HEADER_PATH "\"\n"
+    ".byte 0\n"
+    ".previous\n");
+extern "C" const char kcg_device_src[];
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string& msg) {
+  g_err = msg;
+  return code;
+}
+
+// ---------------------------------------------------------------------------------------------
+// HIP runtime / hiprtc binding.  The library is NOT linked against libamdhip64 / libhiprtc: a
+// process must talk to exactly one HIP runtime, and a host program may already carry its own (the
+// PyTorch wheel bundles one next to libtorch_hip.so).  So the entry points are looked up at first
+// use: an already-loaded libamdhip64.so.7 / libhiprtc.so.7 wins (RTLD_NOLOAD finds it whatever scope
+// it was loaded in); otherwise the system one is opened through this library's RUNPATH.
+// ---------------------------------------------------------------------------------------------
+#define KCG_STR2(x) #x
+#define KCG_STR(x) KCG_STR2(x)
+
+#define KCG_HIP_FUNCS(X)      \
+  X(hipSetDevice)             \
+  X(hipModuleLoadData)        \
+  X(hipModuleGetFunction)     \
+  X(hipModuleUnload)          \
+  X(hipFuncGetAttribute)      \
+  X(hipModuleLaunchKernel)    \
+  X(hipEventCreate)           \
+  X(hipEventRecord)           \
+  X(hipEventSynchronize)      \
+  X(hipEventElapsedTime)      \
+  X(hipEventDestroy)          \
+  X(hipStreamSynchronize)     \
+  X(hipGetDeviceProperties)   \
+  X(hipGetErrorString)
+
+#define KCG_RTC_FUNCS(X)      \
+  X(hiprtcCreateProgram)      \
+  X(hiprtcCompileProgram)     \
+  X(hiprtcGetProgramLogSize)  \
+  X(hiprtcGetProgramLog)      \
+  X(hiprtcGetCodeSize)        \
+  X(hiprtcGetCode)            \
+  X(hiprtcDestroyProgram)     \
+  X(hiprtcGetErrorString)     \
+  X(hiprtcVersion)
+
+struct HipApi {
+#define X(name) decltype(&::name) p_##name = nullptr;
+  KCG_HIP_FUNCS(X)
+#undef X
+  // hipFunction_t overload of hipFuncSetAttribute lives behind the plain C symbol
+  hipError_t (*p_hipFuncSetAttribute)(const void*, hipFuncAttribute, int) = nullptr;
+  std::string error;
+  bool ok = false;
+};
+struct RtcApi {
+#define X(name) decltype(&::name) p_##name = nullptr;
+  KCG_RTC_FUNCS(X)
+#undef X
+  std::string error;
+  bool ok = false;
+};
+
+void* open_shared(const char* soname, std::string* err) {
+  void* h = dlopen(soname, RTLD_NOW | RTLD_NOLOAD);
+  if (!h) h = dlopen(soname, RTLD_NOW | RTLD_LOCAL);
+  if (!h && err) *err = std::string("cannot load ") + soname + ": " + (dlerror() ? dlerror() : "?");
+  return h;
+}
+
+const HipApi& hip_api() {
+  static const HipApi api = [] {
+    HipApi a;
+    void* h = open_shared("libamdhip64.so.7", &a.error);
+    if (!h) return a;
+    bool all = true;
+#define X(name)                                                              \
+  a.p_##name = reinterpret_cast<decltype(&::name)>(dlsym(h, KCG_STR(name))); \
+  if (!a.p_##name) { all = false; a.error += std::string(" missing symbol ") + KCG_STR(name); }
+    KCG_HIP_FUNCS(X)
+#undef X
+    a.p_hipFuncSetAttribute =
+        reinterpret_cast<hipError_t (*)(const void*, hipFuncAttribute, int)>(dlsym(h, "hipFuncSetAttribute"));
+    a.ok = all;
+    return a;
+  }();
+  return api;
+}
+
+const RtcApi& rtc_api() {
+  static const RtcApi api = [] {
+    RtcApi a;
+    void* h = open_shared("libhiprtc.so.7", &a.error);
+    if (!h) return a;
+    bool all = true;
+#define X(name)                                                              \
+  a.p_##name = reinterpret_cast<decltype(&::name)>(dlsym(h, KCG_STR(name))); \
+  if (!a.p_##name) { all = false; a.error += std::string(" missing symbol ") + KCG_STR(name); }
+    KCG_RTC_FUNCS(X)
+#undef X
+    a.ok = all;
+    return a;
+  }();
+  return api;
+}
+
+#define HIPF(name) (hip_api().p_##name)
+#define RTCF(name) (rtc_api().p_##name)
+
+// Same text shape as the reference loader's errors (loaderCCode/hip.c:8-21).
+int hip_fail(hipError_t e, const char* what) {
+  char buf[1024];
+  const char* txt = hip_api().ok ? HIPF(hipGetErrorString)(e) : "?";
+  snprintf(buf, sizeof(buf), "KCG Error[HIP]:  Code: %d, Messsage: %s (%s)", (int)e, txt, what);
+  g_err = buf;
+  return KCG_ERR_HIP;
+}
+
+#define HIP_READY()                                                                         \
+  do {                                                                                      \
+    if (!hip_api().ok) return fail(KCG_ERR_HIP, "KCG Error[HIP]: runtime unavailable:" + hip_api().error); \
+  } while (0)
+
+#define HIP_TRY(expr)                                   \
+  do {                                                  \
+    hipError_t _e = (expr);                             \
+    if (_e != hipSuccess) return hip_fail(_e, #expr);   \
+  } while (0)
+
+uint64_t fnv1a(const std::string& s, uint64_t h = 1469598103934665603ull) {
+  for (unsigned char ch : s) {
+    h ^= ch;
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+bool env_flag(const char* name, bool dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  return !(v[0] == '0' || v[0] == 'n' || v[0] == 'N' || v[0] == 'f' || v[0] == 'F');
+}
+
+std::string library_dir() {
+  Dl_info info;
+  if (dladdr((void*)&kcg_device_src, &info) && info.dli_fname) {
+    std::string p = info.dli_fname;
+    size_t k = p.find_last_of('/');
+    if (k != std::string::npos) return p.substr(0, k);
+  }
+  return ".";
+}
+
+std::string cache_dir() {
+  const char* v = getenv("KCG_CACHE_DIR");
+  if (v && *v) return v;
+  return library_dir() + "/_kcg_cache";
+}
+
+bool make_dirs(const std::string& path) {
+  std::string cur;
+  for (size_t i = 0; i <= path.size(); ++i) {
+    if (i == path.size() || path[i] == '/') {
+      if (!cur.empty()) {
+        if (mkdir(cur.c_str(), 0777) != 0 && errno != EEXIST) return false;
+      }
+    }
+    if (i < path.size()) cur.push_back(path[i]);
+  }
+  return true;
+}
+
+bool file_exists(const std::string& p) {
+  struct stat st;
+  return stat(p.c_str(), &st) == 0 && S_ISREG(st.st_mode) && st.st_size > 0;
+}
+
+bool read_file(const std::string& p, std::vector<char>* out) {
+  FILE* f = fopen(p.c_str(), "rb");
+  if (!f) return false;
+  fseek(f, 0, SEEK_END);
+  long n = ftell(f);
+  rewind(f);
+  out->resize(n > 0 ? n : 0);
+  size_t got = n > 0 ? fread(out->data(), 1, n, f) : 0;
+  fclose(f);
+  return (long)got == n;
+}
+
+// Write-then-rename so that concurrent compile processes never expose a partial code object.
+bool write_file_atomic(const std::string& p, const char* data, size_t n) {
+  static std::atomic<unsigned> counter{0};
+  char suffix[64];
+  snprintf(suffix, sizeof(suffix), ".tmp.%d.%u", (int)getpid(), counter.fetch_add(1));
+  std::string tmp = p + suffix;
+  FILE* f = fopen(tmp.c_str(), "wb");
+  if (!f) return false;
+  size_t w = fwrite(data, 1, n, f);
+  if (fclose(f) != 0 || w != n) {
+    unlink(tmp.c_str());
+    return false;
+  }
+  if (rename(tmp.c_str(), p.c_str()) != 0) {
+    unlink(tmp.c_str());
+    return false;
+  }
+  return true;
+}
+
+const std::vector<std::string>& compile_flags() {
+  static const std::vector<std::string> flags = {
+      "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+  };
+  return flags;
+}
+
+int resolve_kind(const kcg::MatmulConfig& c, int kind, std::string* why) {
+  if (kind == KCG_KIND_SIMT) {
+    *why = kcg::check_simt(c);
+    return why->empty() ? (int)KCG_KIND_SIMT : (int)KCG_ERR_INVALID_CONFIG;
+  }
+  if (kind == KCG_KIND_MFMA) {
+    *why = kcg::check_mfma(c);
+    return why->empty() ? (int)KCG_KIND_MFMA : (int)KCG_ERR_INVALID_CONFIG;
+  }
+  if (kind != KCG_KIND_AUTO) {
+    *why = "unknown kernel kind";
+    return KCG_ERR_ARGUMENT;
+  }
+  std::string wm = kcg::check_mfma(c);
+  if (wm.empty()) return KCG_KIND_MFMA;
+  std::string ws = kcg::check_simt(c);
+  if (ws.empty()) return KCG_KIND_SIMT;
+  *why = "matrix-core kernel: " + wm + "; SIMT kernel: " + ws;
+  return KCG_ERR_INVALID_CONFIG;
+}
+
+int copy_out(const std::string& s, char* out, int out_len) {
+  if (out && out_len > 0) {
+    size_t n = std::min((size_t)out_len - 1, s.size());
+    memcpy(out, s.data(), n);
+    out[n] = 0;
+  }
+  return (int)s.size();
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* kcg_last_error(void) { return g_err.c_str(); }
+const char* kcg_version(void) { return KCG_VERSION; }
+
+const char* kcg_cfg_keyword(int index) {
+  static const char* const kw[KCG_CFG_LEN] = {
+      "BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "THREAD_SIZE_M", "THREAD_SIZE_N", "WARP_SIZE",
+      "BLOCK_LAYOUT_M", "BLOCK_LAYOUT_N", "WARP_LAYOUT_M", "WARP_LAYOUT_N",
+      "GLOB_LOAD_WIDTH_A", "GLOB_LOAD_WIDTH_B", "WARP_SCATTER_WIDTH_A", "WARP_SCATTER_WIDTH_B",
+      "THREAD_SCATTER_WIDTH_A", "THREAD_SCATTER_WIDTH_B", "LOCAL_SPLIT_U", "BLOCK_MAPPING", "GLOB_STORE_WIDTH",
+      "UNROLL_NUM", "REG_PREFETCH", "SHARED_PREFETCH", "LOAD_CONTINUOUS", "REDUCE_C_CONTINUOUS",
+      "DATATYPE_A", "DATATYPE_B", "DATATYPE_C", "M_SIZE", "N_SIZE", "K_SIZE", "IS_ATRANS"};
+  if (index < 0 || index >= KCG_CFG_LEN) return nullptr;
+  return kw[index];
+}
+
+int kcg_dtype_size(int dtype) { return kcg::dtype_size(dtype); }
+
+int kcg_check_config(const kcg_matmul_cfg* cfg, int kind) {
+  if (!cfg) return fail(KCG_ERR_ARGUMENT, "cfg is null");
+  std::string why;
+  int k = resolve_kind(kcg::MatmulConfig::from(*cfg), kind, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  g_err.clear();
+  return KCG_OK;
+}
+
+int kcg_select_kind(const kcg_matmul_cfg* cfg) {
+  if (!cfg) return fail(KCG_ERR_ARGUMENT, "cfg is null");
+  std::string why;
+  int k = resolve_kind(kcg::MatmulConfig::from(*cfg), KCG_KIND_AUTO, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  return k;
+}
+
+int kcg_kernel_name(const kcg_matmul_cfg* cfg, char* out, int out_len) {
+  if (!cfg) return fail(KCG_ERR_ARGUMENT, "cfg is null");
+  return copy_out(kcg::kernel_name(kcg::MatmulConfig::from(*cfg)), out, out_len);
+}
+
+int kcg_launch_dims(const kcg_matmul_cfg* cfg, int32_t grid[3], int32_t block[3]) {
+  if (!cfg || !grid || !block) return fail(KCG_ERR_ARGUMENT, "null argument");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  if (c.BM <= 0 || c.BN <= 0 || c.TM <= 0 || c.TN <= 0) return fail(KCG_ERR_INVALID_CONFIG, "invalid config: tile sizes must be positive");
+  grid[0] = c.grid_y() * c.grid_x();
+  grid[1] = grid[2] = 1;
+  block[0] = c.thread_num();
+  block[1] = block[2] = 1;
+  return KCG_OK;
+}
+
+int kcg_reference_lds_bytes(const kcg_matmul_cfg* cfg) {
+  if (!cfg) return fail(KCG_ERR_ARGUMENT, "cfg is null");
+  return kcg::reference_lds_bytes(kcg::MatmulConfig::from(*cfg));
+}
+
+int kcg_block_mapping(const kcg_matmul_cfg* cfg, int bid, int xcd_remap, int32_t* by, int32_t* bx) {
+  if (!cfg || !by || !bx) return fail(KCG_ERR_ARGUMENT, "null argument");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  if (c.BM <= 0 || c.BN <= 0) return fail(KCG_ERR_INVALID_CONFIG, "invalid config: tile sizes must be positive");
+  if (bid < 0 || bid >= c.grid_x() * c.grid_y()) return fail(KCG_ERR_ARGUMENT, "block id out of range");
+  int y, x;
+  kcg::block_mapping(c, bid, xcd_remap != 0, &y, &x);
+  *by = y;
+  *bx = x;
+  return KCG_OK;
+}
+
+int kcg_instantiation_source(const kcg_matmul_cfg* cfg, int kind, char* out, int out_len) {
+  if (!cfg) return fail(KCG_ERR_ARGUMENT, "cfg is null");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  std::string why;
+  int k = resolve_kind(c, kind, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  return copy_out(kcg::instantiation_source(c, k, env_flag("KCG_XCD_REMAP", true)), out, out_len);
+}
+
+int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, kcg_kernel_info* out) {
+  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  std::string why;
+  int k = resolve_kind(c, kind, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
+  const bool xcd = env_flag("KCG_XCD_REMAP", true);
+  const std::string name = kcg::kernel_name(c);
+  const std::string stub = kcg::instantiation_source(c, k, xcd);
+
+  memset(out, 0, sizeof(*out));
+  if (name.size() >= sizeof(out->kernel_name)) return fail(KCG_ERR_ARGUMENT, "kernel name too long");
+  memcpy(out->kernel_name, name.c_str(), name.size() + 1);
+  out->grid[0] = c.grid_y() * c.grid_x();
+  out->grid[1] = out->grid[2] = 1;
+  out->block[0] = c.thread_num();
+  out->block[1] = out->block[2] = 1;
+  out->lds_bytes = kcg::lds_bytes(c, k);
+  out->kind = k;
+
+  if (!rtc_api().ok) return fail(KCG_ERR_COMPILE, "hiprtc unavailable:" + rtc_api().error);
+  std::string flags_text;
+  for (const auto& f : compile_flags()) flags_text += f + " ";
+  {
+    int major = 0, minor = 0;
+    RTCF(hiprtcVersion)(&major, &minor);
+    flags_text += "hiprtc" + std::to_string(major) + "." + std::to_string(minor);
+  }
+  uint64_t h = fnv1a(KCG_VERSION);
+  h = fnv1a(arch, h);
+  h = fnv1a(flags_text, h);
+  h = fnv1a(stub, h);
+  h = fnv1a(kcg_device_src, h);
+  char hex[32];
+  snprintf(hex, sizeof(hex), "%016llx", (unsigned long long)h);
+
+  const std::string dir = cache_dir();
+  if (!make_dirs(dir)) return fail(KCG_ERR_IO, "cannot create cache directory " + dir);
+  const std::string path = dir + "/" + name + "." + hex + ".hsaco";
+  if (path.size() >= sizeof(out->code_path)) return fail(KCG_ERR_IO, "code object path too long");
+  memcpy(out->code_path, path.c_str(), path.size() + 1);
+
+  if (file_exists(path) && !env_flag("KCG_CACHE_BYPASS", false)) {
+    out->cache_hit = 1;
+    g_err.clear();
+    return KCG_OK;
+  }
+
+  hiprtcProgram prog;
+  const char* hdr_src[] = {kcg_device_src};
+  const char* hdr_name[] = {"kcg_gemm_device.h"};
+  hiprtcResult r = RTCF(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", 1, hdr_src, hdr_name);
+  if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTCF(hiprtcGetErrorString)(r));
+  std::vector<std::string> opts = compile_flags();
+  opts.push_back("--offload-arch=" + arch);
+  std::vector<const char*> optv;
+  for (const auto& o : opts) optv.push_back(o.c_str());
+  r = RTCF(hiprtcCompileProgram)(prog, (int)optv.size(), optv.data());
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    RTCF(hiprtcGetProgramLogSize)(prog, &n);
+    std::string log(n, 0);
+    if (n) RTCF(hiprtcGetProgramLog)(prog, &log[0]);
+    RTCF(hiprtcDestroyProgram)(&prog);
+    return fail(KCG_ERR_COMPILE, std::string("hiprtc: ") + RTCF(hiprtcGetErrorString)(r) + " for " + name + "\n" + log);
+  }
+  size_t n = 0;
+  r = RTCF(hiprtcGetCodeSize)(prog, &n);
+  std::vector<char> code(n);
+  if (r == HIPRTC_SUCCESS) r = RTCF(hiprtcGetCode)(prog, code.data());
+  RTCF(hiprtcDestroyProgram)(&prog);
+  if (r != HIPRTC_SUCCESS || n == 0) return fail(KCG_ERR_COMPILE, "hiprtc returned no code object");
+  if (!write_file_atomic(path, code.data(), code.size())) return fail(KCG_ERR_IO, "cannot write " + path);
+  if (env_flag("KCG_KEEP_SOURCE", false)) {
+    std::string sp = dir + "/" + name + "." + hex + ".hip";
+    write_file_atomic(sp, stub.data(), stub.size());
+  }
+  g_err.clear();
+  return KCG_OK;
+}
+
+int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int device, uint64_t* module,
+             uint64_t* function, int32_t* n_regs, int32_t* n_spills) {
+  if (!code_path || !kernel_name || !module || !function) return fail(KCG_ERR_ARGUMENT, "null argument");
+  std::vector<char> code;
+  if (!read_file(code_path, &code) || code.empty()) return fail(KCG_ERR_IO, std::string("cannot read code object ") + code_path);
+  HIP_READY();
+  HIP_TRY(HIPF(hipSetDevice)(device));
+  hipModule_t mod;
+  hipFunction_t fn;
+  HIP_TRY(HIPF(hipModuleLoadData)(&mod, code.data()));
+  hipError_t e = HIPF(hipModuleGetFunction)(&fn, mod, kernel_name);
+  if (e != hipSuccess) {
+    (void)HIPF(hipModuleUnload)(mod);
+    return hip_fail(e, "hipModuleGetFunction");
+  }
+  if (lds_bytes > 64 * 1024) {
+    e = hip_api().p_hipFuncSetAttribute
+            ? hip_api().p_hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes)
+            : hipErrorNotSupported;
+    if (e != hipSuccess) {
+      (void)HIPF(hipModuleUnload)(mod);
+      return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    }
+  }
+  int regs = 0, local = 0;
+  (void)HIPF(hipFuncGetAttribute)(&regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, fn);
+  (void)HIPF(hipFuncGetAttribute)(&local, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, fn);
+  if (n_regs) *n_regs = regs;
+  if (n_spills) *n_spills = local / 4;   // scratch dwords per lane; 0 means no spilling
+  *module = (uint64_t)(uintptr_t)mod;
+  *function = (uint64_t)(uintptr_t)fn;
+  g_err.clear();
+  return KCG_OK;
+}
+
+int kcg_launch(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes, uint64_t stream,
+               uint64_t a, uint64_t b, uint64_t c) {
+  if (!function || !grid || !block) return fail(KCG_ERR_ARGUMENT, "null function / dims");
+  if ((int64_t)grid[0] * grid[1] * grid[2] <= 0) return KCG_OK;  // empty grid: nothing to do
+  if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
+  void* pa = (void*)(uintptr_t)a;
+  void* pb = (void*)(uintptr_t)b;
+  void* pc = (void*)(uintptr_t)c;
+  void* params[3] = {&pa, &pb, &pc};
+  HIP_READY();
+  HIP_TRY(HIPF(hipModuleLaunchKernel)((hipFunction_t)(uintptr_t)function, grid[0], grid[1], grid[2], block[0], block[1],
+                                block[2], lds_bytes, (hipStream_t)(uintptr_t)stream, params, nullptr));
+  return KCG_OK;
+}
+
+int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes, uint64_t stream,
+                  uint64_t a, uint64_t b, uint64_t c, int warmup, int iters, int reps, float* median_ms,
+                  float* min_ms) {
+  if (iters <= 0) return fail(KCG_ERR_ARGUMENT, "iters must be positive");
+  hipStream_t st = (hipStream_t)(uintptr_t)stream;
+  hipEvent_t e0, e1;
+  HIP_READY();
+  HIP_TRY(HIPF(hipEventCreate)(&e0));
+  HIP_TRY(HIPF(hipEventCreate)(&e1));
+  int rc = KCG_OK;
+  std::vector<float> samples;
+  auto timed = [&](int n, float* ms) -> int {
+    hipError_t e = HIPF(hipEventRecord)(e0, st);
+    if (e != hipSuccess) return hip_fail(e, "hipEventRecord");
+    for (int i = 0; i < n; ++i) {
+      int r = kcg_launch(function, grid, block, lds_bytes, stream, a, b, c);
+      if (r != KCG_OK) return r;
+    }
+    e = HIPF(hipEventRecord)(e1, st);
+    if (e != hipSuccess) return hip_fail(e, "hipEventRecord");
+    e = HIPF(hipEventSynchronize)(e1);
+    if (e != hipSuccess) return hip_fail(e, "hipEventSynchronize");
+    e = HIPF(hipEventElapsedTime)(ms, e0, e1);
+    if (e != hipSuccess) return hip_fail(e, "hipEventElapsedTime");
+    return KCG_OK;
+  };
+  for (int i = 0; i < warmup && rc == KCG_OK; ++i) rc = kcg_launch(function, grid, block, lds_bytes, stream, a, b, c);
+  if (rc == KCG_OK) {
+    hipError_t e = HIPF(hipStreamSynchronize)(st);
+    if (e != hipSuccess) rc = hip_fail(e, "hipStreamSynchronize");
+  }
+  if (rc == KCG_OK && reps <= 0) {
+    float probe = 0.f;
+    rc = timed(1, &probe);
+    if (rc == KCG_OK) {
+      reps = probe > 0.f ? (int)(1.0f / probe) + 1 : 1;
+      if (reps > 1000) reps = 1000;
+    }
+  }
+  for (int i = 0; i < iters && rc == KCG_OK; ++i) {
+    float ms = 0.f;
+    rc = timed(reps, &ms);
+    if (rc == KCG_OK) samples.push_back(ms / (float)reps);
+  }
+  (void)HIPF(hipEventDestroy)(e0);
+  (void)HIPF(hipEventDestroy)(e1);
+  if (rc != KCG_OK) return rc;
+  std::sort(samples.begin(), samples.end());
+  const size_t n = samples.size();
+  if (median_ms) *median_ms = (n % 2) ? samples[n / 2] : 0.5f * (samples[n / 2 - 1] + samples[n / 2]);
+  if (min_ms) *min_ms = samples[0];
+  return KCG_OK;
+}
+
+int kcg_unload(uint64_t module) {
+  if (!module) return fail(KCG_ERR_ARGUMENT, "null module");
+  HIP_READY();
+  HIP_TRY(HIPF(hipModuleUnload)((hipModule_t)(uintptr_t)module));
+  return KCG_OK;
+}
+
+int kcg_device_info(int device, int32_t* cu_count, int32_t* clock_khz, int32_t* lds_per_block, char* arch_name,
+                    int arch_len) {
+  hipDeviceProp_t p;
+  HIP_READY();
+  HIP_TRY(HIPF(hipGetDeviceProperties)(&p, device));
+  if (cu_count) *cu_count = p.multiProcessorCount;
+  if (clock_khz) *clock_khz = p.clockRate;
+  if (lds_per_block) *lds_per_block = (int32_t)p.sharedMemPerBlock;
+  copy_out(p.gcnArchName, arch_name, arch_len);
+  return KCG_OK;
+}
+
+}  // extern "C"

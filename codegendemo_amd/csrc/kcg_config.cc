@@ -1,0 +1,282 @@
+// kcg_config.cc — see kcg_config.h.
+#include "kcg_config.h"
+
+#include <sstream>
+
+namespace kcg {
+
+MatmulConfig MatmulConfig::from(const kcg_matmul_cfg& r) {
+  MatmulConfig c;
+  const int32_t* v = r.v;
+  c.BM = v[KCG_BLOCK_SIZE_M]; c.BN = v[KCG_BLOCK_SIZE_N]; c.BK = v[KCG_BLOCK_SIZE_K];
+  c.TM = v[KCG_THREAD_SIZE_M]; c.TN = v[KCG_THREAD_SIZE_N]; c.WARP_SIZE = v[KCG_WARP_SIZE];
+  c.BLM = v[KCG_BLOCK_LAYOUT_M]; c.BLN = v[KCG_BLOCK_LAYOUT_N];
+  c.WLM = v[KCG_WARP_LAYOUT_M]; c.WLN = v[KCG_WARP_LAYOUT_N];
+  c.GLW_A = v[KCG_GLOB_LOAD_WIDTH_A]; c.GLW_B = v[KCG_GLOB_LOAD_WIDTH_B];
+  c.WSW_A = v[KCG_WARP_SCATTER_WIDTH_A]; c.WSW_B = v[KCG_WARP_SCATTER_WIDTH_B];
+  c.TSW_A = v[KCG_THREAD_SCATTER_WIDTH_A]; c.TSW_B = v[KCG_THREAD_SCATTER_WIDTH_B];
+  c.LSU = v[KCG_LOCAL_SPLIT_U]; c.BLOCK_MAPPING = v[KCG_BLOCK_MAPPING]; c.GSW = v[KCG_GLOB_STORE_WIDTH];
+  c.UNROLL = v[KCG_UNROLL_NUM]; c.REGP = v[KCG_REG_PREFETCH]; c.SHMP = v[KCG_SHARED_PREFETCH];
+  c.LC = v[KCG_LOAD_CONTINUOUS]; c.RC = v[KCG_REDUCE_C_CONTINUOUS];
+  c.dtA = v[KCG_DTYPE_A]; c.dtB = v[KCG_DTYPE_B]; c.dtC = v[KCG_DTYPE_C];
+  c.M = v[KCG_M]; c.N = v[KCG_N]; c.K = v[KCG_K];
+  c.ATRANS = v[KCG_IS_ATRANS];
+  return c;
+}
+
+kcg_matmul_cfg MatmulConfig::raw() const {
+  kcg_matmul_cfg r;
+  int32_t* v = r.v;
+  v[KCG_BLOCK_SIZE_M] = BM; v[KCG_BLOCK_SIZE_N] = BN; v[KCG_BLOCK_SIZE_K] = BK;
+  v[KCG_THREAD_SIZE_M] = TM; v[KCG_THREAD_SIZE_N] = TN; v[KCG_WARP_SIZE] = WARP_SIZE;
+  v[KCG_BLOCK_LAYOUT_M] = BLM; v[KCG_BLOCK_LAYOUT_N] = BLN;
+  v[KCG_WARP_LAYOUT_M] = WLM; v[KCG_WARP_LAYOUT_N] = WLN;
+  v[KCG_GLOB_LOAD_WIDTH_A] = GLW_A; v[KCG_GLOB_LOAD_WIDTH_B] = GLW_B;
+  v[KCG_WARP_SCATTER_WIDTH_A] = WSW_A; v[KCG_WARP_SCATTER_WIDTH_B] = WSW_B;
+  v[KCG_THREAD_SCATTER_WIDTH_A] = TSW_A; v[KCG_THREAD_SCATTER_WIDTH_B] = TSW_B;
+  v[KCG_LOCAL_SPLIT_U] = LSU; v[KCG_BLOCK_MAPPING] = BLOCK_MAPPING; v[KCG_GLOB_STORE_WIDTH] = GSW;
+  v[KCG_UNROLL_NUM] = UNROLL; v[KCG_REG_PREFETCH] = REGP; v[KCG_SHARED_PREFETCH] = SHMP;
+  v[KCG_LOAD_CONTINUOUS] = LC; v[KCG_REDUCE_C_CONTINUOUS] = RC;
+  v[KCG_DTYPE_A] = dtA; v[KCG_DTYPE_B] = dtB; v[KCG_DTYPE_C] = dtC;
+  v[KCG_M] = M; v[KCG_N] = N; v[KCG_K] = K;
+  v[KCG_IS_ATRANS] = ATRANS;
+  return r;
+}
+
+const char* dtype_name(int dt) {
+  switch (dt) {
+    case KCG_DT_FLOAT16: return "float16";
+    case KCG_DT_BFLOAT16: return "bfloat16";
+    case KCG_DT_FLOAT32: return "float32";
+    case KCG_DT_FLOAT64: return "float64";
+    default: return "";
+  }
+}
+
+const char* dtype_ctype(int dt) {
+  switch (dt) {
+    case KCG_DT_FLOAT16: return "_Float16";
+    case KCG_DT_BFLOAT16: return "__bf16";
+    case KCG_DT_FLOAT32: return "float";
+    case KCG_DT_FLOAT64: return "double";
+    default: return "void";
+  }
+}
+
+int dtype_size(int dt) {
+  switch (dt) {
+    case KCG_DT_FLOAT16: return 2;
+    case KCG_DT_BFLOAT16: return 2;
+    case KCG_DT_FLOAT32: return 4;
+    case KCG_DT_FLOAT64: return 8;
+    default: return 0;
+  }
+}
+
+static bool is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+
+static std::string fmt(const char* what, int a) {
+  std::ostringstream s;
+  s << what << " (got " << a << ")";
+  return s.str();
+}
+
+std::string check_common(const MatmulConfig& c) {
+  if (c.M <= 0 || c.N <= 0 || c.K <= 0) return "M_SIZE, N_SIZE, K_SIZE must be positive";
+  if (c.BM <= 0 || c.BN <= 0 || c.BK <= 0) return "BLOCK_SIZE_M/N/K must be positive";
+  if (c.TM <= 0 || c.TN <= 0) return "THREAD_SIZE_M/N must be positive";
+  if (c.WARP_SIZE != 64) return fmt("WARP_SIZE must be 64 on gfx950", c.WARP_SIZE);
+  if (c.BLM <= 0 || c.BLN <= 0 || c.WLM <= 0 || c.WLN <= 0) return "BLOCK_LAYOUT / WARP_LAYOUT must be positive";
+  if (c.WLM * c.WLN != c.WARP_SIZE) return "WARP_LAYOUT_M * WARP_LAYOUT_N != WARP_SIZE";           // matmul.py:190,267-274
+  if (c.BM % c.TM || c.BN % c.TN) return "BLOCK_SIZE_M/N not divisible by THREAD_SIZE_M/N";         // matmul.py:186-187
+  if (c.BLM * c.WLM * c.TM != c.BM) return "BLOCK_LAYOUT_M * WARP_LAYOUT_M * THREAD_SIZE_M != BLOCK_SIZE_M";  // matmul.py:188,300-303
+  if (c.BLN * c.WLN * c.TN != c.BN) return "BLOCK_LAYOUT_N * WARP_LAYOUT_N * THREAD_SIZE_N != BLOCK_SIZE_N";
+  if (c.LSU < 1) return fmt("LOCAL_SPLIT_U must be >= 1", c.LSU);
+  if (c.BK % c.LSU) return "BLOCK_SIZE_K not divisible by LOCAL_SPLIT_U";                          // Optimizer.cc:310
+  if (c.thread_num() > kMaxThreads) return fmt("threads per block exceed 1024", c.thread_num());
+  if (c.BLOCK_MAPPING < 0) return "BLOCK_MAPPING must be >= 0";
+  if (!dtype_size(c.dtA) || !dtype_size(c.dtB) || !dtype_size(c.dtC)) return "unsupported DATATYPE code";
+  if (c.dtA != c.dtB) return "DATATYPE_A and DATATYPE_B must be equal";
+  const bool same = (c.dtC == c.dtA);
+  const bool widen = (c.dtC == KCG_DT_FLOAT32) && (c.dtA == KCG_DT_FLOAT16 || c.dtA == KCG_DT_BFLOAT16);
+  if (!same && !widen) return "DATATYPE_C must equal DATATYPE_A, or be float32 for 16-bit inputs";
+  const int sz = dtype_size(c.dtA);
+  if (!is_pow2(c.GLW_A) || !is_pow2(c.GLW_B)) return "GLOB_LOAD_WIDTH_A/B must be a power of two >= 1";
+  if (c.GLW_A * sz > 16 || c.GLW_B * sz > 16) return "GLOB_LOAD_WIDTH_A/B wider than 128 bits";
+  if (!is_pow2(c.GSW) || c.GSW * dtype_size(c.dtC) > 16) return "GLOB_STORE_WIDTH must be a power of two, at most 128 bits";
+  return "";
+}
+
+int simt_pad_a(const MatmulConfig& c) {
+  if (c.ATRANS) return 0;
+  return c.TSW_A > 4 ? c.TSW_A : 4;
+}
+
+std::string check_simt(const MatmulConfig& c) {
+  std::string e = check_common(c);
+  if (!e.empty()) return e;
+  const int szA = dtype_size(c.dtA);
+  if (!is_pow2(c.TSW_A) || !is_pow2(c.TSW_B) || !is_pow2(c.WSW_A) || !is_pow2(c.WSW_B))
+    return "WARP/THREAD_SCATTER_WIDTH must be powers of two >= 1";
+  if (c.WSW_A < c.TSW_A || c.WSW_B < c.TSW_B) return "WARP_SCATTER_WIDTH < THREAD_SCATTER_WIDTH";     // matmul.py:309-310
+  if (c.WSW_A % c.TSW_A || c.WSW_B % c.TSW_B) return "WARP_SCATTER_WIDTH not a multiple of THREAD_SCATTER_WIDTH";  // matmul.py:311-312
+  if (c.TM % c.WSW_A || c.TN % c.WSW_B) return "THREAD_SIZE not a multiple of WARP_SCATTER_WIDTH";     // Optimizer.cc:21-24
+  if (c.TSW_A * szA > 16 || c.TSW_B * szA > 16 || c.TSW_B * dtype_size(c.dtC) > 16)
+    return "THREAD_SCATTER_WIDTH wider than 128 bits";
+  if (c.ATRANS) {
+    if (c.BM % c.GLW_A) return "BLOCK_SIZE_M not divisible by GLOB_LOAD_WIDTH_A";                   // matmul.cpp:2481-2483
+  } else {
+    if (c.BK % c.GLW_A) return "BLOCK_SIZE_K not divisible by GLOB_LOAD_WIDTH_A (A is [M,K])";
+  }
+  if (c.BN % c.GLW_B) return "BLOCK_SIZE_N not divisible by GLOB_LOAD_WIDTH_B";
+  if (c.LSU > 1 && (c.BN % c.GSW)) return "BLOCK_SIZE_N not divisible by GLOB_STORE_WIDTH";
+  if (c.TM * c.TN > 256) return "thread tile larger than 256 accumulators";
+  if (lds_bytes(c, KCG_KIND_SIMT) > kMaxLdsBytes) return "LDS footprint exceeds 160 KiB";
+  return "";
+}
+
+MfmaPlan plan_mfma(const MatmulConfig& c) {
+  MfmaPlan p;
+  if (c.BLM <= 0 || c.BLN <= 0 || c.BM % c.BLM || c.BN % c.BLN) {
+    p.why = "block tile not divisible by BLOCK_LAYOUT";
+    return p;
+  }
+  p.WM = c.BM / c.BLM;
+  p.WN = c.BN / c.BLN;
+  if (p.WM % 16 || p.WN % 16) {
+    p.why = "wave tile (WARP_LAYOUT*THREAD_SIZE) is not a multiple of the 16x16 matrix-core tile";
+    return p;
+  }
+  p.MF = (p.WM % 32 == 0 && p.WN % 32 == 0) ? 32 : 16;
+  const int sz = dtype_size(c.dtA);
+  if (sz != 2 && sz != 4) {
+    p.why = "matrix-core kernel supports float32, float16 and bfloat16 inputs";
+    return p;
+  }
+  p.G = 16 / sz;
+  p.KS = p.G * (64 / p.MF);
+  p.ok = true;
+  return p;
+}
+
+std::string check_mfma(const MatmulConfig& c) {
+  std::string e = check_common(c);
+  if (!e.empty()) return e;
+  MfmaPlan p = plan_mfma(c);
+  if (!p.ok) return p.why;
+  if (c.BK % (p.KS * c.LSU)) {
+    std::ostringstream s;
+    s << "BLOCK_SIZE_K must be a multiple of " << p.KS << "*LOCAL_SPLIT_U for the " << p.MF << "x" << p.MF
+      << " matrix-core tile";
+    return s.str();
+  }
+  if ((p.WM / p.MF) * (p.WN / p.MF) * (p.MF * p.MF / 64) > 256) return "wave tile needs more than 256 accumulator registers";
+  if (c.LSU > 1 && (c.BN % c.GSW)) return "BLOCK_SIZE_N not divisible by GLOB_STORE_WIDTH";
+  if (lds_bytes(c, KCG_KIND_MFMA) > kMaxLdsBytes) return "LDS footprint exceeds 160 KiB";
+  return "";
+}
+
+// MatmulParams::getKernelName (src/main.cc:119-145)
+std::string kernel_name(const MatmulConfig& c) {
+  std::ostringstream ss;
+  ss << "GEMM_";
+  ss << "MNK" << c.M << "x" << c.N << "x" << c.K << "_";
+  ss << "DTabc" << dtype_name(c.dtA) << "x" << dtype_name(c.dtB) << "x" << dtype_name(c.dtC) << "_";
+  ss << "AT" << c.ATRANS << "_";
+  ss << "TTmn" << c.TM << "x" << c.TN << "_";
+  ss << "BTmnk" << c.BM << "x" << c.BN << "x" << c.BK << "_";
+  ss << "BLmn" << c.BLM << "x" << c.BLN << "_";
+  ss << "WLmn" << c.WLM << "x" << c.WLN << "_";
+  ss << "GLWab" << c.GLW_A << "x" << c.GLW_B << "_";
+  ss << "GSW" << c.GSW << "_";
+  ss << "WSWab" << c.WSW_A << "x" << c.WSW_B << "_";
+  ss << "TSWab" << c.TSW_A << "x" << c.TSW_B << "_";
+  ss << "LSU" << c.LSU << "_";
+  ss << "BM" << c.BLOCK_MAPPING << "_";
+  ss << "UNROLL" << c.UNROLL << "_";
+  ss << "REGP" << c.REGP << "_";
+  ss << "SHMP" << c.SHMP << "_";
+  ss << "LC" << c.LC << "_";
+  ss << "RC" << c.RC << "_";
+  return ss.str();
+}
+
+// UserInputs.sharedMem (CompiledKernelFactory.py:30-44)
+int reference_lds_bytes(const MatmulConfig& c) {
+  int sizeA = c.BM * c.BK * dtype_size(c.dtA);
+  int sizeB = c.BN * c.BK * dtype_size(c.dtB);
+  int sizeAB = sizeA + sizeB;
+  if (c.SHMP > 0) sizeAB *= 2;
+  int sizeC = -1;
+  if (c.LSU > 1) sizeC = c.BM * c.BN * c.LSU * dtype_size(c.dtA);
+  return sizeAB > sizeC ? sizeAB : sizeC;
+}
+
+int lds_bytes(const MatmulConfig& c, int kind) {
+  const int stages = c.SHMP ? 2 : 1;
+  const int szA = dtype_size(c.dtA), szB = dtype_size(c.dtB);
+  const int accsz = (c.dtC == KCG_DT_FLOAT64) ? 8 : 4;
+  int ab;
+  if (kind == KCG_KIND_MFMA) {
+    ab = stages * (c.BM + c.BN) * c.BK * szA;
+  } else {
+    const int lda = c.BM + simt_pad_a(c), ldb = c.BN;
+    const int offB = (stages * c.BK * lda * szA + 15) & ~15;
+    ab = offB + stages * c.BK * ldb * szB;
+  }
+  int cbytes = (c.LSU > 1) ? c.LSU * c.BM * c.BN * accsz : 0;
+  int r = ab > cbytes ? ab : cbytes;
+  return (r + 15) & ~15;
+}
+
+// Rewriter::BlockMapping with isCol=true (Rewriter.cc:726-761; Rewriter.h:112)
+void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int* bx) {
+  const int gy = c.grid_y(), gx = c.grid_x();
+  const int nb = gy * gx;
+  if (xcd_remap && nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
+  const int g = c.BLOCK_MAPPING;
+  if (g > 0 && gy % g == 0) {
+    const int gn = g * gx;
+    *by = (bid / gn) * g + bid % g;
+    *bx = (bid % gn) / g;
+  } else {
+    *by = bid / gx;
+    *bx = bid % gx;
+  }
+}
+
+std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap) {
+  std::ostringstream s;
+  const char* acc = (c.dtC == KCG_DT_FLOAT64) ? "double" : "float";
+  s << "// generated by libkcg_gemm: instantiation of the " << (kind == KCG_KIND_MFMA ? "gemm_mfma" : "gemm_simt")
+    << " template\n";
+  s << "#include \"kcg_gemm_device.h\"\n";
+  s << "namespace {\nstruct Cfg {\n";
+  s << "  typedef " << dtype_ctype(c.dtA) << " TA;\n";
+  s << "  typedef " << dtype_ctype(c.dtB) << " TB;\n";
+  s << "  typedef " << dtype_ctype(c.dtC) << " TC;\n";
+  s << "  typedef " << acc << " ACC;\n";
+  auto I = [&](const char* n, int v) { s << "  static constexpr int " << n << " = " << v << ";\n"; };
+  auto Bv = [&](const char* n, bool v) { s << "  static constexpr bool " << n << " = " << (v ? "true" : "false") << ";\n"; };
+  I("M", c.M); I("N", c.N); I("K", c.K);
+  I("BM", c.BM); I("BN", c.BN); I("BK", c.BK); I("TM", c.TM); I("TN", c.TN);
+  I("WARP_SIZE", c.WARP_SIZE); I("BLM", c.BLM); I("BLN", c.BLN); I("WLM", c.WLM); I("WLN", c.WLN);
+  I("GLW_A", c.GLW_A); I("GLW_B", c.GLW_B); I("WSW_A", c.WSW_A); I("WSW_B", c.WSW_B);
+  I("TSW_A", c.TSW_A); I("TSW_B", c.TSW_B); I("LSU", c.LSU); I("BLOCK_MAPPING", c.BLOCK_MAPPING);
+  I("GSW", c.GSW); I("UNROLL", c.UNROLL);
+  Bv("REGP", c.REGP != 0); Bv("SHMP", c.SHMP != 0);
+  I("LC", c.LC != 0); I("RC", c.RC != 0);
+  Bv("ATRANS", c.ATRANS != 0);
+  Bv("EDGE", c.edge());
+  Bv("XCD_REMAP", xcd_remap);
+  I("SIMT_PAD_A", simt_pad_a(c)); I("SIMT_PAD_B", 0);
+  s << "};\n}  // namespace\n\n";
+  s << "extern \"C\" __global__ __launch_bounds__(" << c.thread_num() << ") void " << kernel_name(c)
+    << "(const Cfg::TA* __restrict__ A, const Cfg::TB* __restrict__ B, Cfg::TC* __restrict__ C) {\n";
+  s << "  extern __shared__ __attribute__((aligned(16))) char kcg_shm0[];\n";
+  s << "  kcg::" << (kind == KCG_KIND_MFMA ? "gemm_mfma" : "gemm_simt") << "<Cfg>(A, B, C, kcg_shm0);\n";
+  s << "}\n";
+  return s.str();
+}
+
+}  // namespace kcg
