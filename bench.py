@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""bench.py — GEMM throughput of the engine on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one pass of the hot path over one batch of synthetic input: one launch of the tuned
+kernel for fp32 C[4096,4096] = A[4096,4096] · B[4096,4096] (row-major A[M,K], B[K,N]; seeded
+uniform[-1,1) inputs already resident in HBM).  The JSON line printed at the end carries
+
+  value / ms_per_step : whole-job throughput over exactly K steps between two device synchronisations
+  roofline            : 2MNK / (average launch duration measured with HIP events on the launch
+                        stream over the same K launches) against the fp32 MFMA peak of MI355X
+  fp16                : the same two figures for the fp16-input / fp32-accumulate kernel at 4096^3
+  cpu_baseline        : the CPU oracle (a port of the reference's hostMatmul arithmetic) timed on this
+                        box's host cores on a bounded row panel of the same product
+
+Only one GPU is ever used; --gpus above 1 exits with a message.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6, "bf16": 2516.6}   # MI355X dense matrix peaks
+HBM_PEAK_GBS = 8000.0
+
+
+def load_tuned(name):
+    with open(os.path.join(ROOT, "codegendemo_amd", "TunedConfigs", name)) as f:
+        return json.load(f)["cfgs"][0]
+
+
+def build_kernel(config):
+    from codegendemo_amd.kcg.CompiledKernelFactory import CompiledKernelFactory, EnumOperator, UserInputs
+    from codegendemo_amd.kcg.KCGCompiler import KCGCompiler
+    from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
+    kpm = kernelArgFromConfig(config)
+    comp = KCGCompiler()
+    path, name, gx, gy, gz, bx, by, bz = comp.compileKernel(kpm)[0]
+    ui = UserInputs(path, name, kpm)
+    ui.m_gridDims, ui.m_blockDims = [gx, gy, gz], [bx, by, bz]
+    ui.m_ldsBytes = comp.lastInfo["lds_bytes"]
+    ui.operatorKind = EnumOperator.Matmul
+    return kpm, CompiledKernelFactory.getKernel(ui, 0), comp.lastInfo
+
+
+def make_inputs(kpm, dist):
+    import torch
+    from codegendemo_amd.kcg import SeededInputs as SI
+    if dist == "uniform":
+        a = SI.uniform((kpm.M, kpm.K), SI.STREAM_A)
+        b = SI.uniform((kpm.K, kpm.N), SI.STREAM_B)
+    else:
+        a = SI.normal((kpm.M, kpm.K), SI.STREAM_A, std=0.5)
+        b = SI.normal((kpm.K, kpm.N), SI.STREAM_B, std=0.5)
+    ta = kpm.dtypeTorch('A')
+    A = torch.from_numpy(SI.a_operand(a, kpm.isATranspose)).to("cuda:0").to(ta)
+    B = torch.from_numpy(b).to("cuda:0").to(ta)
+    C = torch.zeros((kpm.M, kpm.N), dtype=kpm.dtypeTorch('C'), device="cuda:0")
+    return a, b, A, B, C
+
+
+def time_steps(kernel, A, B, C, steps, warmup):
+    """-> (wall ms per step over K steps, HIP-event average launch duration in ms)."""
+    import torch
+    for _ in range(warmup):
+        kernel.run(A, B, C)
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record(stream)               # the kernel is launched on this same (torch current) stream
+    for _ in range(steps):
+        kernel.run(A, B, C)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, ev0.elapsed_time(ev1) / steps
+
+
+def cpu_baseline(a, b, ijk_seconds=8.0):
+    """Times the CPU oracle on this box's host cores: the threaded loop over the WHOLE 4096^3 product
+    (best of 3; it is also the parity reference for the GPU result) and, for the record, the
+    reference's own loop order (i-j-k, one thread) on a row panel sized to a few seconds."""
+    from tests import oracle_binding
+    orc = oracle_binding.load()
+    M, K = a.shape
+    N = b.shape[1]
+    threads = orc.max_threads()
+    best = None
+    full = None
+    spent = 0.0
+    for _ in range(3):
+        t0 = time.perf_counter()
+        full = orc.matmul(a, b, 0)
+        dt = time.perf_counter() - t0
+        spent += dt
+        best = dt if best is None else min(best, dt)
+        if spent > 20.0:
+            break
+    t0 = time.perf_counter()
+    orc.ijk(a, b, 0, rows=(0, 1))
+    probe = time.perf_counter() - t0
+    rows_ijk = int(max(1, min(64, ijk_seconds / max(probe, 1e-4))))
+    t0 = time.perf_counter()
+    orc.ijk(a, b, 0, rows=(0, rows_ijk))
+    dt_ijk = time.perf_counter() - t0
+    return {
+        "value": 2.0 * M * N * K / best / 1e12, "unit": "TFLOPS", "cores": threads, "kind": "port",
+        "sample": f"whole fp32 4096^3 product on the same inputs, best of 3 runs ({best:.2f} s each), "
+                  f"i-k-j loop order, OpenMP over rows",
+        "reference_loop_order": {"value": 2.0 * rows_ijk * N * K / dt_ijk / 1e12, "unit": "TFLOPS", "cores": 1,
+                                 "sample": f"i-j-k order (hostMatmul), first {rows_ijk} rows of C, {dt_ijk:.1f} s"},
+    }, full, M
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-fp16", action="store_true", help="skip the fp16 side measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X; this engine has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from codegendemo_amd import _native
+    _native.lib()   # raises if the native library is missing: there is no fallback
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    cfg32 = load_tuned("gemm_4096_fp32.json")
+    kpm, kernel, info = build_kernel(cfg32)
+    a, b, A, B, C = make_inputs(kpm, "uniform")
+    ms_step, ms_launch = time_steps(kernel, A, B, C, args.steps, args.warmup)
+    flops = 2.0 * kpm.M * kpm.N * kpm.K
+    value = flops / (ms_step * 1e-3) / 1e12
+    achieved = flops / (ms_launch * 1e-3) / 1e12
+    c_host = C.cpu().numpy()
+
+    out = {
+        "metric": "GEMM TFLOPS and % of dtype MFMA roofline at M=N=K=4096, 1 MI355X",
+        "value": value, "unit": "TFLOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fp32 GEMM M=N=K=4096, row-major A[M,K] B[K,N], uniform[-1,1) seeded, tuned config",
+                   "kernel": info["kernel_name"], "kind": {1: "simt", 2: "mfma"}[info["kind"]],
+                   "lds_bytes": info["lds_bytes"], "grid": info["grid"][0], "block": info["block"][0]},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS["f32"], "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_TFLOPS["f32"], "traffic": None,
+                     "launch_ms": ms_launch,
+                     "hbm_gbs_algorithmic": (4.0 * (kpm.M * kpm.K + kpm.K * kpm.N + kpm.M * kpm.N)) / (ms_launch * 1e-3) / 1e9},
+    }
+
+    if not args.no_fp16:
+        cfg16 = load_tuned("gemm_4096_fp16.json")
+        kpm16, kernel16, info16 = build_kernel(cfg16)
+        _, _, A16, B16, C16 = make_inputs(kpm16, "normal")
+        ms_step16, ms_launch16 = time_steps(kernel16, A16, B16, C16, args.steps, args.warmup)
+        ach16 = flops / (ms_launch16 * 1e-3) / 1e12
+        out["fp16"] = {"value": flops / (ms_step16 * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_step16,
+                       "dtype": "f16 in, f32 accumulate/out", "kernel": info16["kernel_name"],
+                       "roofline": {"bound": "mfma", "achieved": ach16, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                                    "frac": ach16 / PEAK_TFLOPS["f16"], "launch_ms": ms_launch16}}
+
+    if not args.no_cpu:
+        base, panel, rows = cpu_baseline(a, b)
+        out["cpu_baseline"] = base
+        err = float(np.abs(c_host[:rows] - panel).max())
+        tol = 1e-4 * kpm.K * float(np.abs(a).max()) * float(np.abs(b).max())
+        out["parity"] = {"rows_checked": rows, "max_abs_err": err, "tolerance": tol, "ok": bool(err <= tol)}
+        if err > tol:
+            print(json.dumps(out))
+            print("bench.py: GPU result differs from the oracle beyond tolerance", file=sys.stderr)
+            sys.exit(1)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

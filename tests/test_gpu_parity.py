@@ -104,6 +104,26 @@ def test_exact_small_integers_16bit(oracle, tag, kw, kind):
     assert bad.size == 0, f"{tag}: {len(bad)} mismatches, first at {bad[:5].tolist()}"
 
 
+def extra_build_configs():
+    """(config, kind) pairs of the full-size tests below, so a build step can precompile them."""
+    out = []
+    for kind in (SIMT, MFMA):
+        for at in (0, 1):
+            out.append((make_config(1024, 1024, 1024, BM=64, BN=64, BK=16, TM=4, TN=4, is_atrans=at), kind))
+    for kind, kw in CONFIG4_KERNELS:
+        out.append((make_config(4096, 1536, 1000, **kw), kind))
+    for kw in CONFIG5_KERNELS:
+        out.append((make_config(4096, 4096, 4096, dtype=2, dtype_c=4, is_atrans=0, **kw), MFMA))
+    return out
+
+
+CONFIG4_KERNELS = ((MFMA, dict(BM=128, BN=128, TM=8, TN=8, BK=16, shared_prefetch=1, is_atrans=0)),
+                   (MFMA, dict(BM=64, BN=64, BK=32, is_atrans=1)),
+                   (SIMT, dict(BM=64, BN=64, BK=8, is_atrans=0)))
+CONFIG5_KERNELS = (dict(BM=128, BN=128, TM=8, TN=8, BK=32, shared_prefetch=1, reg_prefetch=1),
+                   dict(BM=64, BN=64, BK=32))
+
+
 def test_config1_fp32_1024_uniform(oracle):
     """BASELINE config 1: fp32 1024^3, BM=BN=64, BK=16, TM=TN=4, row-major A[M,K], uniform[-1,1)."""
     M = N = K = 1024
@@ -131,10 +151,7 @@ def test_config4_fp32_edge_tiles_normal(oracle):
     rows = (2000, 2096)
     want = oracle.matmul(a, b, a_trans=False, rows=rows)
     tol = fp32_tolerance(K, a, b)
-    for kind, kw in ((MFMA, dict(BM=128, BN=128, TM=8, TN=8, BK=16, shared_prefetch=1)),
-                     (MFMA, dict(BM=64, BN=64, BK=32, is_atrans=1)),
-                     (SIMT, dict(BM=64, BN=64, BK=8))):
-        kw.setdefault("is_atrans", 0)
+    for kind, kw in CONFIG4_KERNELS:
         cfg = make_config(M, N, K, **kw)
         print(f"[case] config4 kind={kind} {kw}", flush=True)
         got, _ = run_gemm(cfg, a, b, kind)
@@ -157,8 +174,7 @@ def test_config5_fp16_4096(oracle):
     rows = (1024, 1088)
     want = oracle.matmul(a, b, a_trans=False, rows=rows)
     scale = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
-    for kw in (dict(BM=128, BN=128, TM=8, TN=8, BK=32, shared_prefetch=1, reg_prefetch=1),
-               dict(BM=64, BN=64, BK=32)):
+    for kw in CONFIG5_KERNELS:
         cfg = make_config(M, N, K, dtype=2, dtype_c=4, is_atrans=0, **kw)
         print(f"[case] config5 {kw}", flush=True)
         got, _ = run_gemm(cfg, a, b, MFMA)
