@@ -105,7 +105,7 @@ class TuningSpaceChecker_Matmul:
         DATATYPE_A/B/C like the reference does (matmul.py:251-265)."""
         kw = ConfigKeywords
         dtypeC = config[kw.KEY_DTYPE_C]
-        nbytes = sizeof(get_dtype_from_int(dtypeC))
+        nbytes = sizeof(get_dtype_from_int(config.get(kw.KEY_DTYPE_A, dtypeC)))   # operands live in LDS
         bm, bn, bk = config[kw.KEY_BLOCK_SIZE_M], config[kw.KEY_BLOCK_SIZE_N], config[kw.KEY_BLOCK_SIZE_K]
         lsu = config[kw.KEY_LOCAL_SPLIT_U]
         stages = 2 if config.get(kw.KEY_SHARED_PREFETCH, 0) else 1

@@ -71,7 +71,7 @@ def a_operand(a_mk, is_a_transposed):
 
 def checksum(x):
     """Order-dependent 64-bit checksum of an array's bytes (for input fixtures)."""
-    b = np.ascontiguousarray(x).view(np.uint8)
+    b = np.ascontiguousarray(x).reshape(-1).view(np.uint8)
     pad = (-b.size) % 8
     if pad:
         b = np.concatenate([b, np.zeros(pad, np.uint8)])

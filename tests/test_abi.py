@@ -1,0 +1,92 @@
+"""The C ABI itself: every function include/kcg_gemm.h declares is exported by libkcg_gemm.so, the
+struct layouts agree, and the entry points that need a GPU fail cleanly (status + message) without one.
+No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from codegendemo_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    with open(os.path.join(ROOT, "include", "kcg_gemm.h")) as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kcg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    names = declared_functions()
+    assert len(names) >= 17
+    lib = _native.lib()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/kcg_gemm.h but not exported"
+    assert set(names) == set(_native.EXPORTS)
+
+
+def test_library_does_not_link_a_hip_runtime():
+    """HIP is bound lazily so the process keeps a single runtime (the host program's)."""
+    import subprocess
+    out = subprocess.run(["readelf", "-d", _native.LIB_PATH], capture_output=True, text=True).stdout
+    needed = re.findall(r"NEEDED.*\[(.*?)\]", out)
+    assert not [n for n in needed if "amdhip" in n or "hiprtc" in n or "torch" in n], needed
+
+
+def test_struct_layouts():
+    assert ctypes.sizeof(_native.MatmulCfg) == 31 * 4
+    assert ctypes.sizeof(_native.KernelInfo) == 1024 + 512 + 4 * (3 + 3 + 3)
+    assert _native.lib().kcg_dtype_size(2) == 2 and _native.lib().kcg_dtype_size(3) == 2
+    assert _native.lib().kcg_dtype_size(4) == 4 and _native.lib().kcg_dtype_size(8) == 8
+    assert _native.lib().kcg_dtype_size(99) == 0
+    assert _native.lib().kcg_cfg_keyword(31) is None and _native.lib().kcg_cfg_keyword(-1) is None
+
+
+def test_error_channel_without_gpu():
+    lib = _native.lib()
+    # missing code object: IO error, message names the path (reference: fopen NULL -> silent NULL, hip.c:79-81)
+    with pytest.raises(_native.KcgError) as ei:
+        _native.load("/nonexistent/kernel.hsaco", "k", 0, 0)
+    assert ei.value.status == _native.ERR_IO and "/nonexistent/kernel.hsaco" in str(ei.value)
+    # null handles / null pointers
+    with pytest.raises(_native.KcgError) as ei:
+        _native.launch(0, [1, 1, 1], [64, 1, 1], 0, 0, 1, 2, 3)
+    assert ei.value.status == _native.ERR_ARGUMENT
+    assert lib.kcg_check_config(None, 0) == _native.ERR_ARGUMENT
+    assert lib.kcg_compile_matmul(None, b"gfx950", 0, None) == _native.ERR_ARGUMENT
+    with pytest.raises(_native.KcgError):
+        _native.unload(0)
+    with pytest.raises(_native.KcgError) as ei:
+        _native.benchmark(1, [1, 1, 1], [64, 1, 1], 0, 0, 1, 2, 3, iters=0)
+    assert ei.value.status == _native.ERR_ARGUMENT
+    # unknown kernel kind
+    from codegendemo_amd.kcg.ConfigGenerator import make_config
+    from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
+    v = kernelArgFromConfig(make_config(256, 256, 128)).values()
+    with pytest.raises(_native.KcgError) as ei:
+        _native.compile_matmul(v, kind=7)
+    assert ei.value.status == _native.ERR_ARGUMENT
+
+
+def test_empty_grid_launch_is_a_no_op():
+    """HIPLauncher.py:138: a launch with an empty grid is skipped."""
+    _native.launch(1234, [0, 1, 1], [64, 1, 1], 0, 0, 1, 2, 3)
+
+
+def test_last_error_is_per_thread():
+    import threading
+    lib = _native.lib()
+    lib.kcg_check_config(None, 0)
+    assert _native.last_error() != ""
+    seen = {}
+
+    def worker():
+        seen["msg"] = _native.last_error()
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert seen["msg"] == ""

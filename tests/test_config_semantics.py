@@ -1,0 +1,192 @@
+"""Host-side config semantics of libkcg_gemm.so (no GPU): keyword table, kernel name, launch
+geometry, LDS bytes, block swizzle, validity — pinned by the reference's own data files and by the
+worked examples in its sources (cited per test)."""
+import itertools
+
+import pytest
+
+from codegendemo_amd import _native
+from codegendemo_amd.kcg.ConfigGenerator import make_config
+from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
+from codegendemo_amd.kcg.Utils import ConfigKeywords
+from tests import fixtures
+
+
+def vals(cfg):
+    return kernelArgFromConfig(cfg).values()
+
+
+def test_keyword_table_matches_reference_files():
+    """Every tuning JSON the reference ships uses exactly the engine's 31 keywords."""
+    kws = set(_native.keywords())
+    assert len(kws) == 31
+    for cfg in fixtures.best_combs_1024():
+        assert set(cfg.keys()) == kws
+    for name, space in fixtures.tuning_spaces().items():
+        assert set(space.keys()) == kws, name
+
+
+def test_abi_order_is_compile_kernel_matmul_order():
+    """src/main.cc:64-96: tile sizes, layouts, load widths, scatter widths, LSU, mapping, store width,
+    unroll + four flags, dtypes, sizes, IS_ATRANS."""
+    o = _native.keywords()
+    assert o[:10] == ["BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "THREAD_SIZE_M", "THREAD_SIZE_N", "WARP_SIZE",
+                      "BLOCK_LAYOUT_M", "BLOCK_LAYOUT_N", "WARP_LAYOUT_M", "WARP_LAYOUT_N"]
+    assert o[10:19] == ["GLOB_LOAD_WIDTH_A", "GLOB_LOAD_WIDTH_B", "WARP_SCATTER_WIDTH_A", "WARP_SCATTER_WIDTH_B",
+                        "THREAD_SCATTER_WIDTH_A", "THREAD_SCATTER_WIDTH_B", "LOCAL_SPLIT_U", "BLOCK_MAPPING",
+                        "GLOB_STORE_WIDTH"]
+    assert o[19:24] == ["UNROLL_NUM", "REG_PREFETCH", "SHARED_PREFETCH", "LOAD_CONTINUOUS", "REDUCE_C_CONTINUOUS"]
+    assert o[24:] == ["DATATYPE_A", "DATATYPE_B", "DATATYPE_C", "M_SIZE", "N_SIZE", "K_SIZE", "IS_ATRANS"]
+
+
+def test_kernel_name_reproduces_reference_sample():
+    """The name in the reference's IR dump (temp.mlir:3) must come out byte for byte
+    (format: src/main.cc:119-145)."""
+    want = fixtures.kernel_name_sample()
+    cfg = make_config(1024, 1024, 1024, BM=32, BN=32, BK=8, TM=4, TN=4, is_atrans=1, glw=4, scatter=2, gsw=4,
+                      block_mapping=16, unroll=1, shared_prefetch=1, reg_prefetch=0, load_continuous=0,
+                      reduce_c_continuous=0)
+    assert _native.kernel_name(vals(cfg)) == want
+
+
+def test_kernel_name_is_injective_over_best_combs():
+    names = {_native.kernel_name(vals(c)) for c in fixtures.best_combs_1024()}
+    assert len(names) == len({tuple(vals(c)) for c in fixtures.best_combs_1024()})
+
+
+def test_launch_dims_worked_example():
+    """matmul.cpp:2392-2413,2448-2449: M=1024, N=1056, BM=64, BN=48, TM=4, TN=6, LSU=2 ->
+    grid (1024/64)*(1056/48) = 16*22, block (64/4)*(48/6)*2 = 256."""
+    cfg = make_config(1024, 1056, 1024, BM=64, BN=48, BK=32, TM=4, TN=6, lsu=2, glw=2, scatter=2, gsw=2)
+    grid, block = _native.launch_dims(vals(cfg))
+    assert grid == [16 * 22, 1, 1] and block == [256, 1, 1]
+
+
+def test_launch_dims_round_up_for_edge_tiles():
+    cfg = make_config(4096, 1536, 1000, BM=128, BN=128, BK=16, TM=8, TN=8)
+    grid, block = _native.launch_dims(vals(cfg))
+    assert grid == [32 * 12, 1, 1] and block == [256, 1, 1]
+    cfg = make_config(130, 70, 9, BM=64, BN=64, BK=16)
+    assert _native.launch_dims(vals(cfg))[0] == [3 * 2, 1, 1]
+
+
+def test_reference_lds_formula():
+    """CompiledKernelFactory.py:30-44: (BM*BK + BN*BK)*size, doubled with SHARED_PREFETCH; with split-U
+    the larger of that and BM*BN*LSU*size."""
+    c = make_config(1024, 1024, 1024, BM=64, BN=64, BK=16)
+    assert _native.reference_lds_bytes(vals(c)) == (64 + 64) * 16 * 4
+    c = make_config(1024, 1024, 1024, BM=64, BN=64, BK=16, shared_prefetch=1)
+    assert _native.reference_lds_bytes(vals(c)) == 2 * (64 + 64) * 16 * 4
+    c = make_config(1024, 1024, 1024, BM=64, BN=64, BK=16, lsu=2)
+    assert _native.reference_lds_bytes(vals(c)) == 64 * 64 * 2 * 4
+    c = make_config(1024, 1024, 1024, BM=128, BN=128, BK=32, TM=8, TN=8, dtype=2, dtype_c=4, shared_prefetch=1)
+    assert _native.reference_lds_bytes(vals(c)) == 2 * (128 + 128) * 32 * 2
+    # the matrix-core kernel needs exactly the reference's operand footprint (no padding)
+    info = _native.compile_matmul(vals(c), kind=_native.KIND_MFMA)
+    assert info["lds_bytes"] == 2 * (128 + 128) * 32 * 2
+
+
+@pytest.mark.parametrize("M,N,BM,BN,G", [(1024, 1024, 64, 64, 8), (1024, 1024, 32, 64, 16), (512, 384, 64, 64, 4),
+                                          (512, 384, 64, 64, 3), (4096, 1536, 128, 128, 8), (200, 136, 64, 64, 8),
+                                          (1024, 1024, 64, 64, 0)])
+@pytest.mark.parametrize("xcd", [0, 1])
+def test_block_mapping_is_a_permutation(M, N, BM, BN, G, xcd):
+    tsz = {32: 4, 64: 4, 128: 8}
+    cfg = make_config(M, N, 64, BM=BM, BN=BN, BK=16, TM=tsz[BM], TN=tsz[BN], block_mapping=G)
+    gy, gx = -(-M // BM), -(-N // BN)
+    seen = {_native.block_mapping(vals(cfg), b, xcd) for b in range(gy * gx)}
+    assert seen == set(itertools.product(range(gy), range(gx)))
+
+
+def test_block_mapping_formula():
+    """Rewriter.cc:726-761 (isCol=true): G = BLOCK_MAPPING, H = N/BN;
+    by = (bid / (G*H))*G + bid % G, bx = (bid % (G*H)) / G when (M/BM) % G == 0, identity otherwise."""
+    cfg = make_config(1024, 1024, 64, BM=64, BN=64, block_mapping=8)      # 16 x 16 blocks
+    v = vals(cfg)
+    for bid in (0, 1, 7, 8, 9, 127, 128, 129, 255):
+        by, bx = _native.block_mapping(v, bid)
+        assert (by, bx) == ((bid // 128) * 8 + bid % 8, (bid % 128) // 8)
+    cfg = make_config(1024, 1024, 64, BM=64, BN=64, block_mapping=5)      # 16 % 5 != 0 -> identity
+    v = vals(cfg)
+    for bid in (0, 1, 17, 255):
+        assert _native.block_mapping(v, bid) == (bid // 16, bid % 16)
+    with pytest.raises(_native.KcgError):
+        _native.block_mapping(v, 256)
+
+
+def test_all_reference_tuned_configs_are_valid_and_select_a_kernel():
+    """The 270 configs of best_combs_1024.json ran correctly on the authors' hardware; the engine must
+    accept every one of them."""
+    kinds = {1: 0, 2: 0}
+    for cfg in fixtures.best_combs_1024():
+        v = vals(cfg)
+        _native.check_config(v)
+        assert _native.is_valid_config(v, _native.KIND_SIMT), cfg     # the literal kernel takes them all
+        kinds[_native.select_kind(v)] += 1
+    assert kinds[1] + kinds[2] == 270
+    assert kinds[2] > 0     # some wave tiles are matrix-core tileable
+
+
+def test_invalid_configs_are_reported_not_compiled():
+    good = make_config(1024, 1024, 1024)
+    cases = {
+        "WARP_LAYOUT": dict(good, WARP_LAYOUT_M=4),                        # 4*8 != 64
+        "BLOCK_LAYOUT_M": dict(good, BLOCK_LAYOUT_M=1),                    # 1*8*4 != 64
+        "LOCAL_SPLIT_U": dict(good, LOCAL_SPLIT_U=3),                      # 16 % 3
+        "WARP_SIZE": dict(good, WARP_SIZE=32, WARP_LAYOUT_M=4),
+        "GLOB_LOAD_WIDTH": dict(good, GLOB_LOAD_WIDTH_A=0),
+        "DATATYPE": dict(good, DATATYPE_A=2),                              # A != B
+        "positive": dict(good, K_SIZE=0),
+        "1024": dict(make_config(1024, 1024, 1024, BM=256, BN=256, BK=16, TM=8, TN=8), LOCAL_SPLIT_U=2),
+    }
+    for needle, cfg in cases.items():
+        v = vals(cfg)
+        assert not _native.is_valid_config(v)
+        with pytest.raises(_native.InvalidConfigError) as ei:
+            _native.compile_matmul(v)
+        assert needle in str(ei.value), (needle, str(ei.value))
+
+
+def test_kind_selection_rules():
+    v = vals(make_config(1024, 1024, 1024, BM=64, BN=64, BK=16))          # 32x32 wave tile, BK%8 == 0
+    assert _native.select_kind(v) == _native.KIND_MFMA
+    v = vals(make_config(1024, 1024, 1024, BM=32, BN=64, BK=8, warp_layout=(4, 16)))   # 16x16 tiles need BK%16
+    assert _native.select_kind(v) == _native.KIND_SIMT
+    v = vals(make_config(1024, 1024, 1024, BM=64, BN=48, BK=32, TM=4, TN=6, scatter=2, glw=2, gsw=2))  # 32x48 wave tile
+    assert _native.select_kind(v) == _native.KIND_MFMA                      # 32x48 wave tile = 2x3 tiles of 16x16
+    v = vals(make_config(512, 512, 512, dtype=8, BM=64, BN=64, BK=16, glw=2, gsw=2, scatter=2))         # fp64: SIMT only
+    assert _native.select_kind(v) == _native.KIND_SIMT
+
+
+def test_instantiation_source_carries_the_config():
+    cfg = make_config(4096, 1536, 1000, BM=128, BN=128, BK=16, TM=8, TN=8, is_atrans=0, shared_prefetch=1)
+    src = _native.instantiation_source(vals(cfg), _native.KIND_MFMA)
+    assert "gemm_mfma<Cfg>" in src and "static constexpr int BM = 128;" in src
+    assert "static constexpr bool EDGE = true;" in src and "static constexpr bool ATRANS = false;" in src
+    assert _native.kernel_name(vals(cfg)) in src
+    assert "__launch_bounds__(256)" in src
+
+
+def test_compile_cache_hit_and_code_object(tmp_path, monkeypatch):
+    monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path / "cache"))
+    v = vals(make_config(256, 256, 128))
+    first = _native.compile_matmul(v)
+    assert not first["cache_hit"]
+    second = _native.compile_matmul(v)
+    assert second["cache_hit"] and second["code_path"] == first["code_path"]
+    with open(first["code_path"], "rb") as f:
+        blob = f.read()
+    assert blob[:4] == b"\x7fELF"
+    assert first["kernel_name"].encode() in blob          # the kernel symbol is the reference kernel name
+    other = _native.compile_matmul(v, kind=_native.KIND_SIMT)
+    assert other["code_path"] != first["code_path"] and other["kernel_name"] == first["kernel_name"]
+
+
+def test_sample_of_reference_tuned_configs_compile(tmp_path, monkeypatch):
+    monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path / "cache"))
+    cfgs = fixtures.best_combs_1024()
+    for cfg in cfgs[::27]:
+        info = _native.compile_matmul(vals(cfg))
+        assert info["block"][0] == (cfg["BLOCK_SIZE_M"] // cfg["THREAD_SIZE_M"]) * \
+            (cfg["BLOCK_SIZE_N"] // cfg["THREAD_SIZE_N"]) * cfg["LOCAL_SPLIT_U"]
+        assert info["grid"][0] == (1024 // cfg["BLOCK_SIZE_M"]) * (1024 // cfg["BLOCK_SIZE_N"])

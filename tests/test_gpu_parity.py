@@ -61,6 +61,8 @@ EXACT_CASES = [
     ("mfma-edge-at0", MFMA, dict(M=200, N=136, K=100, is_atrans=0, shared_prefetch=1)),
     ("mfma-odd", MFMA, dict(M=131, N=67, K=37, is_atrans=0)),
     ("mfma-odd-at1", MFMA, dict(M=131, N=67, K=37, is_atrans=1, lsu=2, BK=32)),
+    ("mfma-64x48", MFMA, dict(M=256, N=192, K=128, BM=64, BN=48, BK=32, TM=4, TN=6, scatter=2, glw=2, gsw=2, lsu=2)),
+    ("simt-64x48", SIMT, dict(M=256, N=192, K=128, BM=64, BN=48, BK=32, TM=4, TN=6, scatter=2, glw=2, gsw=2, lsu=2)),
     ("mfma-bm0", MFMA, dict(M=512, N=256, K=64, block_mapping=0)),
     ("mfma-bm4", MFMA, dict(M=512, N=384, K=64, block_mapping=4)),
 ]

@@ -1,0 +1,175 @@
+"""The Python operator API mirrors the reference's kcg package: same records, same JSON, same call
+shapes (CPU only)."""
+import json
+import os
+import pickle
+
+import numpy as np
+import pytest
+
+from codegendemo_amd import _native
+from codegendemo_amd.kcg import SeededInputs as SI
+from codegendemo_amd.kcg.CompiledKernelFactory import CompiledKernelFactory, EnumOperator, UserInputs
+from codegendemo_amd.kcg.ConfigGenerator import config_gen, get_cfgs, iter_cfgs, make_config
+from codegendemo_amd.kcg.KCGCompiler import KCGCompiler
+from codegendemo_amd.kcg.Operators.matmul import (KernelArgMatmul, TuningSpaceChecker_Matmul, getMatmulSignature,
+                                                  kernelArgFromConfig)
+from codegendemo_amd.kcg.Utils import ConfigKeywords, EnumKernelDType, PathManager, ToTorchType, sizeof
+from tests import fixtures
+
+
+def test_enum_codes_and_sizes():
+    """Utils.py:198-221 / Utils.h:110-120: float16=2, float32=4, float64=8; sizeof = code % 30."""
+    assert int(EnumKernelDType.float16) == 2 and int(EnumKernelDType.float32) == 4 and int(EnumKernelDType.float64) == 8
+    assert sizeof(EnumKernelDType.float32) == 4 and sizeof(EnumKernelDType.float16) == 2
+    assert sizeof(EnumKernelDType.int32) == 4 and sizeof(EnumKernelDType.bfloat16) == 2
+    import torch
+    assert ToTorchType(EnumKernelDType.float16) is torch.float16
+    assert ToTorchType(4) is torch.float32 and ToTorchType(3) is torch.bfloat16
+
+
+def test_kernel_arg_defaults_follow_the_reference_constructor():
+    """matmul.py:77-108."""
+    k = KernelArgMatmul(1024, 512, 256, EnumKernelDType.float32, EnumKernelDType.float32, EnumKernelDType.float32)
+    assert (k.BLOCK_SIZE_M, k.BLOCK_SIZE_N, k.BLOCK_SIZE_K, k.THREAD_SIZE_M, k.THREAD_SIZE_N) == (64, 64, 16, 4, 4)
+    assert (k.WARP_SIZE, k.BLOCK_LAYOUT_M, k.BLOCK_LAYOUT_N, k.WARP_LAYOUT_M, k.WARP_LAYOUT_N) == (64, 4, 1, 16, 4)
+    assert (k.M, k.N, k.K, k.isATranspose, k.UNROLL_NUM) == (1024, 512, 256, 1, 1)
+    assert k.GLOB_LOAD_WIDTH_A == 0 and k.LOCAL_SPLIT_U == 0 and k.SHARED_PREFETCH == 0
+    assert k.dtype('A') == 4 and k.dtypeTorch('C') is ToTorchType(4)
+
+
+def test_json_round_trip_over_reference_configs():
+    for cfg in fixtures.best_combs_1024()[::9]:
+        k = kernelArgFromConfig(cfg)
+        j = k.jsonfy()
+        assert j == cfg
+        assert list(j.keys()) == list(cfg.keys())      # same key order as the reference writes
+        k2 = KernelArgMatmul(0, 0, 0, 1, 1, 1)
+        k2.assignWithJson(json.loads(json.dumps(j)))
+        assert k2 == k and k2.values() == k.values()
+        json.loads(str(k))                              # __str__ is JSON text like the reference's
+
+
+def test_values_are_in_abi_order():
+    cfg = fixtures.best_combs_1024()[3]
+    k = kernelArgFromConfig(cfg)
+    assert k.values() == [cfg[kw] for kw in _native.keywords()]
+
+
+def test_check_raises_with_reason():
+    k = kernelArgFromConfig(make_config(1024, 1024, 1024))
+    k.check()
+    k.WARP_LAYOUT_N = 4
+    with pytest.raises(ValueError):
+        k.check()
+
+
+def test_signature():
+    import torch
+    assert getMatmulSignature(torch.float32, torch.float32, torch.float32) == {0: "*fp32", 1: "*fp32", 2: "*fp32"}
+    assert getMatmulSignature(torch.float16, torch.float16, torch.float32) == {0: "*fp16", 1: "*fp16", 2: "*fp32"}
+
+
+def test_compiler_return_shape_and_factory(tmp_path, monkeypatch):
+    """compile_kernel_matmul returns [(path, name, gx, gy, gz, bx, by, bz)] (src/main.cc:335-348)."""
+    monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path / "c"))
+    kpm = kernelArgFromConfig(make_config(1024, 1024, 1024, shared_prefetch=1))
+    res = KCGCompiler().compileKernel(kpm)
+    assert isinstance(res, list) and len(res) == 1 and len(res[0]) == 8
+    path, name, gx, gy, gz, bx, by, bz = res[0]
+    assert os.path.isfile(path) and name.startswith("GEMM_MNK1024x1024x1024_DTabcfloat32xfloat32xfloat32_AT1_")
+    assert (gx, gy, gz, bx, by, bz) == (256, 1, 1, 256, 1, 1)
+    assert KCGCompiler().compile_kernel_matmul(*kpm.values()) == res
+    ui = UserInputs(path, name, kpm)
+    assert ui.sharedMem() == 2 * (64 + 64) * 16 * 4       # reference formula when the engine value is unknown
+    ui.m_gridDims, ui.m_blockDims = [gx, gy, gz], [bx, by, bz]
+    assert ui.numCTA() == 256 and ui.operatorKind == EnumOperator.Matmul
+    kernel = CompiledKernelFactory.getKernel(ui, 0)
+    assert kernel.signature == {0: "*fp32", 1: "*fp32", 2: "*fp32"}
+    # picklable before first run, handles never travel (KCGTask.py:305-318)
+    kernel._module, kernel._function = 11, 22
+    k2 = pickle.loads(pickle.dumps((kpm, ui, kernel)))[2]
+    assert k2._function == 0 and k2.kernelBinaryPath == path and k2.gridDims == [256, 1, 1]
+    with pytest.raises(TypeError):
+        k2.run(1, 2)
+
+
+def test_tuning_space_checkers():
+    chk = TuningSpaceChecker_Matmul
+    good = make_config(1024, 1024, 1024)
+    assert chk.check_warp(dict(good)) and chk.check_size(dict(good)) and chk.check_shm_size(dict(good))
+    assert not chk.check_warp(dict(good, WARP_LAYOUT_M=4))
+    assert not chk.check_size(dict(good, BLOCK_LAYOUT_M=1))
+    assert not chk.check_size(dict(good, WARP_SCATTER_WIDTH_A=1, THREAD_SCATTER_WIDTH_A=2))
+    assert chk.check_size(dict(good, K_SIZE=1000))                               # edge tiles are allowed here …
+    assert not chk.check_size(dict(good, K_SIZE=1000), allow_edge_tiles=False)   # … the reference rule rejects them
+    big = make_config(4096, 4096, 4096, BM=256, BN=256, BK=64, TM=8, TN=8, dtype=2, dtype_c=4, shared_prefetch=1)
+    assert chk.check_shm_size(dict(big))                                         # 128 KiB fits gfx950's 160 KiB
+    assert not chk.check_shm_size(dict(big, BLOCK_SIZE_K=128))
+    # DATATYPE_C alone is expanded to A/B (matmul.py:259-263)
+    c = {k: v for k, v in good.items() if k not in ("DATATYPE_A", "DATATYPE_B")}
+    assert chk.check_shm_size(c) and c["DATATYPE_A"] == 4 and c["DATATYPE_B"] == 4
+
+
+def test_get_cfgs_on_reference_tuning_space():
+    """GEMM_single_test.json describes one point; GEMM_configs_1024.json a large space whose every
+    emitted point must pass the engine predicate."""
+    spaces = fixtures.tuning_spaces()
+    single = list(iter_cfgs(spaces["GEMM_single_test.json"]))
+    assert len(single) == 1 and single[0]["BLOCK_SIZE_N"] == 64 and single[0]["WARP_LAYOUT_N"] == 16
+    space = dict(spaces["GEMM_configs_1024.json"])
+    for k in ("UNROLL_NUM", "BLOCK_MAPPING", "GLOB_STORE_WIDTH", "REDUCE_C_CONTINUOUS", "LOAD_CONTINUOUS",
+              "WARP_SCATTER_WIDTH_A", "WARP_SCATTER_WIDTH_B", "THREAD_SCATTER_WIDTH_A", "THREAD_SCATTER_WIDTH_B"):
+        space[k] = space[k][:1]      # keep the enumeration small for a unit test
+    stats = {}
+    cfgs = list(iter_cfgs(space, stats=stats))
+    assert 0 < len(cfgs) < stats["enumerated"]
+    for c in cfgs[::17]:
+        assert _native.is_valid_config([c[k] for k in ConfigKeywords.ORDER])
+
+
+def test_config_gen_splits_into_sub_jsons(tmp_path, monkeypatch):
+    monkeypatch.setenv("KCG_WORK_DIR", str(tmp_path / "work"))
+    PathManager.init(clearTmp=True)
+    space = {k: [v] for k, v in make_config(2048, 2048, 2048).items()}
+    space["BLOCK_SIZE_K"] = [8, 16, 32]
+    space["SHARED_PREFETCH"] = [0, 1]
+    tuning = tmp_path / "space.json"
+    tuning.write_text(json.dumps(space))
+    cache = tmp_path / "combs.json"
+    names, total = config_gen(str(tuning), "", 4, str(cache), splitBigJson=True)
+    assert total == 6 and len(names) == 2
+    assert [len(json.load(open(n))["cfgs"]) for n in names] == [4, 2]
+    assert len(json.load(open(cache))["cfgs"]) == 6
+    names2, total2 = config_gen("", str(cache), 6, "", splitBigJson=True)      # reuse the pre-generated file
+    assert total2 == 6 and len(names2) == 1
+    assert get_cfgs(str(tuning))[0]["M_SIZE"] == 2048
+
+
+def test_seeded_inputs_are_deterministic_and_well_formed():
+    u1 = SI.uniform((64, 48), SI.STREAM_A)
+    u2 = SI.uniform((64, 48), SI.STREAM_A)
+    assert np.array_equal(u1, u2) and u1.dtype == np.float32
+    assert not np.array_equal(u1, SI.uniform((64, 48), SI.STREAM_B))
+    assert u1.min() >= -1.0 and u1.max() < 1.0
+    assert np.array_equal(SI.uniform((4096,), 1)[:100], SI.uniform((100,), 1))      # counter-based: prefix-stable
+    # fixture: integer-exact stream, must never change across machines or numpy versions
+    assert SI.checksum(SI.uniform((1024, 1024), SI.STREAM_A)) == SI.checksum(SI.uniform((1024 * 1024,), SI.STREAM_A))
+    big = SI.uniform((1 << 20,), 7)
+    assert abs(float(big.mean())) < 5e-3 and abs(float(big.var()) - 1.0 / 3.0) < 5e-3
+    n = SI.normal((1 << 20,), 8, std=0.5)
+    assert abs(float(n.mean())) < 5e-3 and abs(float(n.std()) - 0.5) < 5e-3
+    s = SI.small_ints((1000,), 9, lim=4)
+    assert set(np.unique(s)).issubset(set(np.arange(-4, 5, dtype=np.float32))) and len(np.unique(s)) == 9
+    a = SI.uniform((5, 7), 3)
+    assert SI.a_operand(a, 1).shape == (7, 5) and np.array_equal(SI.a_operand(a, 1), a.T)
+
+
+def test_uniform_stream_golden_values():
+    """First values of stream A, committed so the generator cannot drift silently."""
+    got = SI.raw_bits(4, SI.STREAM_A).tolist()
+    with open(os.path.join(fixtures.GOLDEN, "seeded_inputs.json")) as f:
+        want = json.load(f)
+    assert got == want["raw_bits_stream1_first4"]
+    assert SI.checksum(SI.uniform((256, 256), SI.STREAM_A)) == want["checksum_uniform_256x256_stream1"]
+    assert SI.checksum(SI.uniform((256, 256), SI.STREAM_B)) == want["checksum_uniform_256x256_stream2"]
