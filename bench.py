@@ -31,7 +31,8 @@ HBM_PEAK_GBS = 8000.0
 
 
 def load_tuned(name):
-    with open(os.path.join(ROOT, "codegendemo_amd", "TunedConfigs", name)) as f:
+    path = name if os.path.isabs(name) or os.path.exists(name) else os.path.join(ROOT, "codegendemo_amd", "TunedConfigs", name)
+    with open(path) as f:
         return json.load(f)["cfgs"][0]
 
 
@@ -124,9 +125,13 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-fp16", action="store_true", help="skip the fp16 side measurement")
+    ap.add_argument("--fp32-config", default="", help="JSON file ({'cfgs': [...]}) to use instead of the tuned fp32 config")
+    ap.add_argument("--fp16-config", default="", help="same for the fp16 side measurement")
+    ap.add_argument("--only-fp16", action="store_true",
+                    help="profiling aid: run only the fp16 kernel (prints a reduced JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X; this engine has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -140,7 +145,17 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
-    cfg32 = load_tuned("gemm_4096_fp32.json")
+    if args.only_fp16:
+        cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
+        kpm16, kernel16, info16 = build_kernel(cfg16)
+        _, _, A16, B16, C16 = make_inputs(kpm16, "normal")
+        ms_step16, ms_launch16 = time_steps(kernel16, A16, B16, C16, args.steps, args.warmup)
+        fl = 2.0 * kpm16.M * kpm16.N * kpm16.K
+        print(json.dumps({"only": "fp16", "kernel": info16["kernel_name"], "launch_ms": ms_launch16,
+                          "tflops": fl / (ms_launch16 * 1e-3) / 1e12}))
+        return
+
+    cfg32 = load_tuned(args.fp32_config or "gemm_4096_fp32.json")
     kpm, kernel, info = build_kernel(cfg32)
     a, b, A, B, C = make_inputs(kpm, "uniform")
     ms_step, ms_launch = time_steps(kernel, A, B, C, args.steps, args.warmup)
@@ -164,7 +179,7 @@ def main():
     }
 
     if not args.no_fp16:
-        cfg16 = load_tuned("gemm_4096_fp16.json")
+        cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
         kpm16, kernel16, info16 = build_kernel(cfg16)
         _, _, A16, B16, C16 = make_inputs(kpm16, "normal")
         ms_step16, ms_launch16 = time_steps(kernel16, A16, B16, C16, args.steps, args.warmup)

@@ -253,6 +253,26 @@ const std::vector<std::string>& compile_flags() {
   return flags;
 }
 
+// Extra hiprtc options from $KCG_EXTRA_FLAGS (space separated), e.g. "-DNAME=1" or "-save-temps";
+// part of the cache key.  The reference had a comparable hook for injecting an LLVM pass plugin
+// (AMDGCN_INSTRUMENTATION_LIB, LLVMIRTranslation.cc:98-108).
+std::vector<std::string> extra_flags() {
+  std::vector<std::string> out;
+  const char* v = getenv("KCG_EXTRA_FLAGS");
+  if (!v) return out;
+  std::string cur;
+  for (const char* p = v;; ++p) {
+    if (*p == ' ' || *p == 0) {
+      if (!cur.empty()) out.push_back(cur);
+      cur.clear();
+      if (*p == 0) break;
+    } else {
+      cur.push_back(*p);
+    }
+  }
+  return out;
+}
+
 int resolve_kind(const kcg::MatmulConfig& c, int kind, std::string* why) {
   if (kind == KCG_KIND_SIMT) {
     *why = kcg::check_simt(c);
@@ -392,6 +412,7 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
     RTCF(hiprtcVersion)(&major, &minor);
     flags_text += "hiprtc" + std::to_string(major) + "." + std::to_string(minor);
   }
+  for (const auto& f : extra_flags()) flags_text += f + " ";
   uint64_t h = fnv1a(KCG_VERSION);
   h = fnv1a(arch, h);
   h = fnv1a(flags_text, h);
@@ -419,6 +440,7 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTCF(hiprtcGetErrorString)(r));
   std::vector<std::string> opts = compile_flags();
   opts.push_back("--offload-arch=" + arch);
+  for (const auto& f : extra_flags()) opts.push_back(f);
   std::vector<const char*> optv;
   for (const auto& o : opts) optv.push_back(o.c_str());
   r = RTCF(hiprtcCompileProgram)(prog, (int)optv.size(), optv.data());

@@ -173,6 +173,7 @@ std::string check_mfma(const MatmulConfig& c) {
   if ((p.WM / p.MF) * (p.WN / p.MF) * (p.MF * p.MF / 64) > 256) return "wave tile needs more than 256 accumulator registers";
   if (c.LSU > 1 && (c.BN % c.GSW)) return "BLOCK_SIZE_N not divisible by GLOB_STORE_WIDTH";
   if (lds_bytes(c, KCG_KIND_MFMA) > kMaxLdsBytes) return "LDS footprint exceeds 160 KiB";
+  if ((c.SHMP ? 2 : 1) * (c.BM + c.BN) * c.BK * dtype_size(c.dtA) > kMaxLdsBytes) return "LDS footprint exceeds 160 KiB";
   return "";
 }
 
@@ -212,7 +213,26 @@ int reference_lds_bytes(const MatmulConfig& c) {
   return sizeAB > sizeC ? sizeAB : sizeC;
 }
 
+// Must state the same rule as DirectPlan<C>::ELIGIBLE in kcg_gemm_device.h (a static_assert there
+// compares the two): 16-bit inputs, no edge tiles, both prefetch flags, LOAD_CONTINUOUS, 128-bit load
+// widths, power-of-two tiles that split evenly into 1 KiB wave fetches, at least 4 matrix-core groups
+// per K tile, and both LDS stages within 160 KiB.
+bool mfma_direct(const MatmulConfig& c) {
+  MfmaPlan p = plan_mfma(c);
+  if (!p.ok || dtype_size(c.dtA) != 2) return false;
+  if (c.edge() || !c.SHMP || !c.REGP || !c.LC || c.LSU != 1 || c.GLW_A != 8 || c.GLW_B != 8) return false;
+  const int ks = 8 * (64 / p.MF);
+  if (c.BK % ks) return false;
+  const int spw = c.BK / ks, nm = (p.WM / p.MF) * (p.WN / p.MF), nw = c.BLM * c.BLN;
+  if (spw * nm < 4) return false;
+  if (!is_pow2(c.BM) || !is_pow2(c.BN) || !is_pow2(c.BK) || c.BM < 64 || c.BN < 64) return false;
+  if ((c.BM * c.BK / 8) % (64 * nw) || (c.BN * c.BK / 8) % (64 * nw)) return false;
+  if (c.M % 8 || c.N % 8 || c.K % 8) return false;
+  return 2 * (c.BM + c.BN) * c.BK * 2 <= kMaxLdsBytes;
+}
+
 int lds_bytes(const MatmulConfig& c, int kind) {
+  if (kind == KCG_KIND_MFMA && mfma_direct(c)) return 0;   // that path declares its stages statically
   const int stages = c.SHMP ? 2 : 1;
   const int szA = dtype_size(c.dtA), szB = dtype_size(c.dtB);
   const int accsz = (c.dtC == KCG_DT_FLOAT64) ? 8 : 4;
@@ -269,6 +289,7 @@ std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap
   Bv("ATRANS", c.ATRANS != 0);
   Bv("EDGE", c.edge());
   Bv("XCD_REMAP", xcd_remap);
+  Bv("DIRECT", kind == KCG_KIND_MFMA && mfma_direct(c));
   I("SIMT_PAD_A", simt_pad_a(c)); I("SIMT_PAD_B", 0);
   s << "};\n}  // namespace\n\n";
   s << "extern \"C\" __global__ __launch_bounds__(" << c.thread_num() << ") void " << kernel_name(c)

@@ -53,6 +53,7 @@ std::string check_mfma(const MatmulConfig& c);
 std::string kernel_name(const MatmulConfig& c);
 int reference_lds_bytes(const MatmulConfig& c);
 int simt_pad_a(const MatmulConfig& c);
+bool mfma_direct(const MatmulConfig& c);      // matrix-core kernel stages operands with direct global->LDS loads
 int lds_bytes(const MatmulConfig& c, int kind);  // what the chosen kernel family really needs
 void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int* bx);
 

@@ -49,6 +49,7 @@ constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int cmin(int a, int b) { return a < b ? a : b; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 constexpr int lowbit(int a) { return a & (-a); }
+template <bool B> struct BoolC { static constexpr bool value = B; };
 
 // Copy NBYTES (power of two, <= 16) between two suitably aligned addresses as one access.
 template <int NBYTES>
@@ -106,6 +107,29 @@ struct TileMap {
       c = it * (TPR * VEC) + (tid % TPR) * VEC;
       return true;
     }
+  }
+};
+
+// Thread -> (k chunk, first row) map for an operand tile that is contiguous along m/n in global memory
+// and is transposed into [row][k chunk] LDS layout: NCH k-chunks x NVEC row vectors of VEC rows.
+//   ROWS_FAST=1: consecutive threads take consecutive row vectors (widest global coalescing)
+//   ROWS_FAST=0: consecutive threads take consecutive k chunks of one row vector, so the 16-byte LDS
+//                writes of 8 neighbouring lanes land in 8 different bank groups
+template <int NCH, int NVEC, int VEC, int NT, bool ROWS_FAST>
+struct BlockMap {
+  static constexpr int NB = NCH * NVEC;
+  static constexpr int ITERS = cdiv(NB, NT);
+  static constexpr bool FULL = (NB % NT == 0);
+  __device__ __forceinline__ static bool coords(int tid, int it, int& chunk, int& row) {
+    int v = tid + it * NT;
+    if constexpr (ROWS_FAST) {
+      chunk = v / NVEC;
+      row = (v % NVEC) * VEC;
+    } else {
+      chunk = v % NCH;
+      row = (v / NCH) * VEC;
+    }
+    return FULL || v < NB;
   }
 };
 
@@ -454,18 +478,267 @@ template <> struct Mfma<__bf16, 16> {
   }
 };
 
-// LDS operand tile: ROWS rows (m or n) of CH 16-byte chunks (k).  Chunk c of row r lives at chunk
-// slot r*CH + (c ^ swz(r)); swz makes 8 consecutive rows hit 8 different 16-byte bank groups.
+// LDS operand tile: rows (m or n) of CH 16-byte chunks (k).  The LDS of gfx950 has 64 dword banks, i.e.
+// 16 bank groups of 16 bytes; a 128-bit access of a wave costs as many passes as the largest number
+// of lanes (out of every 16) that meet in one group.  Chunk c of row r lives at chunk slot
+// r*CH + (c ^ swz(r)); swz is chosen so that 16 consecutive rows at equal c (a fragment read) fall
+// into 16 different groups.
 template <int CH>
 struct LdsTile {
-  static constexpr int SMOD = cmin(8, lowbit(CH));
-  static constexpr int RDIV = cmax(1, 8 / SMOD);
+  static constexpr int SMOD = cmin(16, lowbit(CH));
+  static constexpr int RDIV = cmax(1, 16 / SMOD);
   __device__ __forceinline__ static int slot(int r, int c) { return r * CH + (c ^ ((r / RDIV) % SMOD)); }
 };
+
+// =============================================================================================
+// Family 2b: matrix-core kernel with direct global->LDS staging (16-bit inputs).
+//
+// Every lane fetches one 16-byte chunk with global_load_lds_dwordx4; a wave's 64 chunks land in 1 KiB of
+// consecutive LDS, so no register, no ds_write and no VALU work is spent on staging and the fetch of
+// tile kt+2 can be in flight for a whole K tile.  The LDS image keeps the orientation of global memory:
+//   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/8 chunks of 8 k values each; a fragment
+//                                           is one ds_read_b128 (as in gemm_mfma)
+//   row-contiguous operand (B; A^T)       : rows = k, NCH = BN/8 (BM/8) chunks of 8 n values each; a
+//                                           fragment is two ds_read_b64_tr_b16: 16 lanes read a 4(k) x
+//                                           16(n) block and each lane receives one column of it, which
+//                                           is the k-packed layout the matrix core wants
+// The bank swizzle is applied on the fetch side: the lane that fills physical chunk c' of a row fetches
+// logical chunk c' ^ swz(row), and readers look chunk c up at c ^ swz(row).
+// =============================================================================================
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+template <class C>
+struct DirectPlan {
+  typedef typename C::TA T;
+  static constexpr int ES = (int)sizeof(T);
+  static constexpr int WM = C::BM / C::BLM, WN = C::BN / C::BLN;
+  static constexpr int MF = (WM % 32 == 0 && WN % 32 == 0) ? 32 : 16;
+  static constexpr int KS = 8 * (64 / MF);
+  static constexpr int NW = C::BLM * C::BLN;
+  static constexpr int NM = (WM / MF) * (WN / MF);
+  static constexpr int SPW = (C::BK % KS == 0) ? C::BK / KS : 0;
+  static constexpr bool pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+  static constexpr bool ELIGIBLE =
+      ES == 2 && !C::EDGE && C::SHMP && C::REGP && C::LC != 0 && C::LSU == 1 && C::GLW_A == 8 && C::GLW_B == 8 &&
+      SPW > 0 && SPW * NM >= 4 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
+      (C::BM * C::BK / 8) % (64 * NW) == 0 && (C::BN * C::BK / 8) % (64 * NW) == 0 && (C::M % 8 == 0) &&
+      (C::N % 8 == 0) && (C::K % 8 == 0) && 2 * (C::BM + C::BN) * C::BK * 2 <= 160 * 1024;
+  // the host picks the path (it must size dynamic LDS accordingly); both sides have to agree
+  static_assert(ELIGIBLE == C::DIRECT, "host and device disagree on the direct-staging eligibility rule");
+  static constexpr bool OK = C::DIRECT;
+};
+
+template <class C>
+__device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
+                                                 typename C::TC* __restrict__ Cm, char* smem) {
+  typedef typename C::TA T;
+  typedef typename C::TC TC;
+  typedef DirectPlan<C> P;
+  constexpr int BM = C::BM, BN = C::BN, BK = C::BK;
+  constexpr int M = C::M, N = C::N, K = C::K;
+  constexpr int WM = P::WM, WN = P::WN, MF = P::MF;
+  constexpr int KH = 64 / MF, KS = P::KS, SPW = P::SPW;
+  constexpr int TMI = WM / MF, TNI = WN / MF, NM = P::NM, NW = P::NW;
+  constexpr int KT = K / BK;
+  constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
+  constexpr int CHK = BK / 8;                           // chunks per row of a k-contiguous tile
+  constexpr int NCHA = BM / 8, NCHB = BN / 8;           // chunks per row of a row-contiguous tile
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int NIA = (BM * BK / 8) / (64 * NW);        // fetch instructions per wave and tile, operand A
+  constexpr int NIB = (BN * BK / 8) / (64 * NW);
+  typedef Mfma<T, MF> MI;
+  typedef typename MI::Acc Acc;
+  typedef typename MI::Frag Frag;
+  typedef LdsTile<CHK> LK;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int wy = wave / C::BLN, wx = wave % C::BLN;
+  int by, bx;
+  block_coords<C>(blockIdx.x, by, bx);
+  const int m0 = by * BM, n0 = bx * BN;
+
+  // The two stages are separate LDS objects on purpose: the compiler then knows that a fragment read
+  // from one stage cannot alias an in-flight fetch into the other and does not wait for the fetch.
+  // (For the same reason the K loop below is unrolled by two, so every access names its stage.)
+  __shared__ __attribute__((aligned(1024))) char lds_stage0[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char lds_stage1[STAGE_BYTES];
+  (void)smem;
+
+  // swizzle of a row-contiguous tile: rows k..k+3 of a transposing read must not share banks
+  auto swz_n = [](int k, int nch) { return ((k & 3) << 2) & (nch - 1); };
+
+  // ---- fetch: global -> LDS ------------------------------------------------------------------
+  auto fetch_item = [&](int idx, int kt, auto stage_c) {
+    char* st = decltype(stage_c)::value ? lds_stage1 : lds_stage0;
+    const int k0 = kt * BK;
+    if (idx < NIA) {
+      const int s = 64 * (wave * NIA + idx) + lane;   // physical chunk slot inside the A stage
+      const T* src;
+      if constexpr (AK) {
+        const int row = s / CHK, cp = s % CHK;
+        const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
+        src = A + (long)(m0 + row) * K + k0 + c * 8;
+      } else {
+        const int k = s / NCHA, cp = s % NCHA;
+        const int c = cp ^ swz_n(k, NCHA);
+        src = A + (long)(k0 + k) * M + m0 + c * 8;
+      }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + 1024 * (wave * NIA + idx)), 16, 0, 0);
+    } else {
+      const int j = idx - NIA;
+      const int s = 64 * (wave * NIB + j) + lane;
+      const int k = s / NCHB, cp = s % NCHB;
+      const int c = cp ^ swz_n(k, NCHB);
+      const T* src = B + (long)(k0 + k) * N + n0 + c * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + A_BYTES + 1024 * (wave * NIB + j)), 16, 0, 0);
+    }
+  };
+  constexpr int NFETCH = NIA + NIB;
+
+  // ---- fragments -----------------------------------------------------------------------------
+  const int frow = lane % MF, fgrp = lane / MF;
+  const int tx = lane % 16;                          // lane inside its 16-lane transposing group
+  const int tsub = (lane / 16) % (MF / 16);          // which 16-column half of the MFMA tile
+  // row-contiguous tile: 8 k values of column (rowbase + lane%MF), k = kb .. kb+7, from two 4x16 blocks
+  // The transposing read is issued as inline assembly: as a builtin the compiler cannot tell that it
+  // does not touch the stage a fetch is in flight to, and would drain all fetches (vmcnt(0)) in front
+  // of every such read.  The price: the compiler does not know these reads are asynchronous either,
+  // so the loop below waits for them itself (wait_tr) before the matrix-core step that consumes them.
+  auto read_tr = [&](const char* tile, int nch, int rowbase, int kb, Frag* dst) {
+    const int n = rowbase + 16 * tsub + 4 * (tx % 4);
+    u32x2 part[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int k = kb + 4 * t + tx / 4;
+      const unsigned addr = (unsigned)(unsigned long)(tile + ((k * nch + ((n / 8) ^ swz_n(k, nch))) * 16) + (n % 8) * 2);
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(part[t]) : "v"(addr));
+    }
+    copy_bytes<16>(dst, part);
+  };
+  // lgkmcnt(0): every LDS read issued so far (compiler-visible or not) has returned
+  auto wait_tr = [&]() { __builtin_amdgcn_s_waitcnt(0xC07F); };
+  auto load_frag_item = [&](auto stage_c, int s, int f, Frag* fa, Frag* fb) {
+    const char* st = decltype(stage_c)::value ? lds_stage1 : lds_stage0;
+    if (f < TMI) {
+      if constexpr (AK) {
+        const int row = wy * WM + f * MF + frow;
+        copy_bytes<16>(&fa[f], st + LK::slot(row, s * KH + fgrp) * 16);
+      } else {
+        read_tr(st, NCHA, wy * WM + f * MF, s * KS + 8 * fgrp, &fa[f]);
+      }
+    } else {
+      read_tr(st + A_BYTES, NCHB, wx * WN + (f - TMI) * MF, s * KS + 8 * fgrp, &fb[f - TMI]);
+    }
+  };
+  constexpr int NF = TMI + TNI;
+
+  Acc acc[TMI][TNI];
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j)
+#pragma unroll
+      for (int e = 0; e < (int)(sizeof(Acc) / sizeof(float)); ++e) acc[i][j][e] = 0.0f;
+
+  // ---- K loop: two LDS stages; the barrier stands in the middle of the last step of a tile --------
+  constexpr int MT = SPW * NM;
+  constexpr int BAR = (SPW - 1) * NM + NM / 2;
+  constexpr int FSPAN = cmax(1, (NM * 3) / 4);
+  constexpr int NSPAN = cmax(1, ((MT - BAR) * 3) / 4);
+  constexpr int TAIL = MT - BAR;
+
+#pragma unroll
+  for (int i = 0; i < NFETCH; ++i) fetch_item(i, 0, BoolC<false>());
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's chunks of tile 0 are in LDS
+  __syncthreads();
+  if (KT > 1) {
+#pragma unroll
+    for (int i = 0; i < NFETCH; ++i) fetch_item(i, 1, BoolC<true>());
+  }
+  Frag fa[2][TMI], fb[2][TNI];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) load_frag_item(BoolC<false>(), 0, f, fa[0], fb[0]);
+
+  // one K tile; `cur_c` is the stage it computes from, has1/has2: tiles kt+1 / kt+2 exist
+  auto tile = [&](int kt, auto cur_c, auto has1, auto has2) {
+    constexpr bool CUR = decltype(cur_c)::value;
+    constexpr bool H1 = decltype(has1)::value, H2 = decltype(has2)::value;
+#pragma unroll
+    for (int s = 0; s < SPW; ++s) {
+#pragma unroll
+      for (int q = 0; q < NM; ++q) {
+        const int slot = s * NM + q;
+        if (slot == BAR) {
+          if constexpr (H1) __builtin_amdgcn_s_waitcnt(0x0F70);   // tile kt+1 has landed (this wave's part)
+          __syncthreads();                                        // ... everyone's part; stage CUR is free
+        }
+        if (q == 0) wait_tr();   // fragments of this step (read under the previous step) are complete
+        MI::run(acc[q / TNI][q % TNI], fa[s & 1][q / TNI], fb[s & 1][q % TNI]);
+        if constexpr (H2) {
+#pragma unroll
+          for (int i = 0; i < NFETCH; ++i)
+            if (BAR + (i * TAIL) / NFETCH == slot) fetch_item(i, kt + 2, BoolC<CUR>());
+        }
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          if (s + 1 < SPW && (f * FSPAN) / NF == q)
+            load_frag_item(BoolC<CUR>(), s + 1, f, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+          if (H1 && BAR + (f * NSPAN) / NF == slot) load_frag_item(BoolC<!CUR>(), 0, f, fa[SPW & 1], fb[SPW & 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (SPW % 2 == 1) {
+#pragma unroll
+      for (int i = 0; i < TMI; ++i) fa[0][i] = fa[1][i];
+#pragma unroll
+      for (int j = 0; j < TNI; ++j) fb[0][j] = fb[1][j];
+    }
+  };
+  typedef BoolC<true> Yes;
+  typedef BoolC<false> No;
+  int kt = 0;
+  for (; kt + 3 < KT; kt += 2) {
+    tile(kt, No(), Yes(), Yes());
+    tile(kt + 1, Yes(), Yes(), Yes());
+  }
+  if (KT - kt == 3) {
+    tile(kt, No(), Yes(), Yes());
+    tile(kt + 1, Yes(), Yes(), No());
+    tile(kt + 2, No(), No(), No());
+  } else if (KT - kt == 2) {
+    tile(kt, No(), Yes(), No());
+    tile(kt + 1, Yes(), No(), No());
+  } else {
+    tile(kt, No(), No(), No());
+  }
+
+  // ---- epilogue (accumulator layout as in gemm_mfma) ---------------------------------------------
+  constexpr int NACC = (int)(sizeof(Acc) / sizeof(float));
+  const int ocol = lane % MF;
+  const int orow = (lane / MF) * 4;
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j)
+#pragma unroll
+      for (int e = 0; e < NACC; ++e) {
+        const int row = m0 + wy * WM + i * MF + (e / 4) * 8 + orow + e % 4;
+        const int col = n0 + wx * WN + j * MF + ocol;
+        Cm[(long)row * N + col] = (TC)acc[i][j][e];
+      }
+}
 
 template <class C>
 __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
                                           typename C::TC* __restrict__ Cm, char* smem) {
+  if constexpr (DirectPlan<C>::OK) {
+    gemm_mfma_direct<C>(A, B, Cm, smem);
+    return;
+  }
   typedef typename C::TA T;   // TA == TB for this family
   typedef typename C::TC TC;
   constexpr int BM = C::BM, BN = C::BN, BK = C::BK, LSU = C::LSU;
@@ -509,8 +782,8 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
   // loads G row vectors, transposes them in registers and writes VEC chunks.
   constexpr int VN_A = cmin(C::GLW_A, G);
   constexpr int VN_B = cmin(C::GLW_B, G);
-  typedef TileMap<CH, BM, VN_A, NT, true> MapNA;
-  typedef TileMap<CH, BN, VN_B, NT, true> MapNB;
+  typedef BlockMap<CH, BM / VN_A, VN_A, NT, C::LC != 0> MapNA;
+  typedef BlockMap<CH, BN / VN_B, VN_B, NT, C::LC != 0> MapNB;
   constexpr int ITERS_A = C::ATRANS ? MapNA::ITERS : MapKA::ITERS;
   constexpr int REGS_A = C::ATRANS ? G * VN_A : G;
   constexpr bool AL_A = C::ATRANS ? (M % VN_A == 0) : (K % VK_A == 0);
@@ -519,68 +792,73 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
   T ga[ITERS_A][REGS_A];
   T gb[MapNB::ITERS][G * VN_B];
 
-  auto load_global = [&](int kt) {
-    const int k0 = kt * BK;
-#pragma unroll
-    for (int it = 0; it < ITERS_A; ++it) {
-      int r, c;
-      if constexpr (C::ATRANS) {
-        if (MapNA::coords(tid, it, r, c)) {   // r = k chunk, c = first m of the vector
-#pragma unroll
-          for (int g = 0; g < G; ++g)
-            gload<T, VN_A, EDGE, AL_A>(&ga[it][g * VN_A], A, k0 + r * G + g, m0 + c, M, K, M);
-        }
-      } else {
-        if (MapKA::coords(tid, it, r, c)) {   // r = m row, c = first k of the chunk
-#pragma unroll
-          for (int v = 0; v < G / VK_A; ++v)
-            gload<T, VK_A, EDGE, AL_A>(&ga[it][v * VK_A], A, m0 + r, k0 + c + v * VK_A, K, M, K);
-        }
+  // The staging work of one K tile is cut into items (one global vector load, or one 16-byte LDS
+  // write, each) so that the pipelined loop below can place them one by one between matrix-core
+  // instructions.  `idx` is a compile-time constant wherever these are called (unrolled loops).
+  constexpr int LPA = C::ATRANS ? G : G / VK_A;   // global loads per A iteration
+  constexpr int WPA = C::ATRANS ? VN_A : 1;       // LDS writes per A iteration
+  constexpr int NLD_A = ITERS_A * LPA, NLD = NLD_A + MapNB::ITERS * G;
+  constexpr int NWR_A = ITERS_A * WPA, NWR = NWR_A + MapNB::ITERS * VN_B;
+
+  auto load_item = [&](int idx, int k0) {
+    int r, c;
+#ifdef KCG_DBG_SAMETILE
+    k0 = 0;
+#endif
+#ifdef KCG_DBG_NOLOAD
+    return;
+#endif
+    if (idx < NLD_A) {
+      const int it = idx / LPA, sub = idx % LPA;
+      if constexpr (C::ATRANS) {   // r = k chunk, c = first m of the vector
+        if (MapNA::coords(tid, it, r, c))
+          gload<T, VN_A, EDGE, AL_A>(&ga[it][sub * VN_A], A, k0 + r * G + sub, m0 + c, M, K, M);
+      } else {                     // r = m row, c = first k of the chunk
+        if (MapKA::coords(tid, it, r, c))
+          gload<T, VK_A, EDGE, AL_A>(&ga[it][sub * VK_A], A, m0 + r, k0 + c + sub * VK_A, K, M, K);
       }
-    }
-#pragma unroll
-    for (int it = 0; it < MapNB::ITERS; ++it) {
-      int r, c;
-      if (MapNB::coords(tid, it, r, c)) {
-#pragma unroll
-        for (int g = 0; g < G; ++g)
-          gload<T, VN_B, EDGE, AL_B>(&gb[it][g * VN_B], B, k0 + r * G + g, n0 + c, N, K, N);
-      }
+    } else {
+      const int it = (idx - NLD_A) / G, sub = (idx - NLD_A) % G;
+      if (MapNB::coords(tid, it, r, c))
+        gload<T, VN_B, EDGE, AL_B>(&gb[it][sub * VN_B], B, k0 + r * G + sub, n0 + c, N, K, N);
     }
   };
-  auto store_lds = [&](int stage) {
+  auto write_item = [&](int idx, int stage) {
+#ifdef KCG_DBG_NOWRITE
+    return;
+#endif
     u32x4* sa = smA + stage * BM * CH;
     u32x4* sb = smB + stage * BN * CH;
-#pragma unroll
-    for (int it = 0; it < ITERS_A; ++it) {
-      int r, c;
+    int r, c;
+    if (idx < NWR_A) {
+      const int it = idx / WPA, e = idx % WPA;
       if constexpr (C::ATRANS) {
         if (MapNA::coords(tid, it, r, c)) {
+          T chunk[G];
 #pragma unroll
-          for (int e = 0; e < VN_A; ++e) {
-            T chunk[G];
-#pragma unroll
-            for (int g = 0; g < G; ++g) chunk[g] = ga[it][g * VN_A + e];
-            copy_bytes<16>(sa + L::slot(c + e, r), chunk);
-          }
+          for (int g = 0; g < G; ++g) chunk[g] = ga[it][g * VN_A + e];
+          copy_bytes<16>(sa + L::slot(c + e, r), chunk);
         }
       } else {
         if (MapKA::coords(tid, it, r, c)) copy_bytes<16>(sa + L::slot(r, c / G), ga[it]);
       }
-    }
-#pragma unroll
-    for (int it = 0; it < MapNB::ITERS; ++it) {
-      int r, c;
+    } else {
+      const int it = (idx - NWR_A) / VN_B, e = (idx - NWR_A) % VN_B;
       if (MapNB::coords(tid, it, r, c)) {
+        T chunk[G];
 #pragma unroll
-        for (int e = 0; e < VN_B; ++e) {
-          T chunk[G];
-#pragma unroll
-          for (int g = 0; g < G; ++g) chunk[g] = gb[it][g * VN_B + e];
-          copy_bytes<16>(sb + L::slot(c + e, r), chunk);
-        }
+        for (int g = 0; g < G; ++g) chunk[g] = gb[it][g * VN_B + e];
+        copy_bytes<16>(sb + L::slot(c + e, r), chunk);
       }
     }
+  };
+  auto load_global = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) load_item(i, kt * BK);
+  };
+  auto store_lds = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < NWR; ++i) write_item(i, stage);
   };
 
   // ---- fragments and matrix-core steps -------------------------------------------------------
@@ -603,6 +881,17 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
 #pragma unroll
     for (int j = 0; j < TNI; ++j) copy_bytes<16>(&fb[j], sb + L::slot(wx * WN + j * MF + frow, c));
   };
+  // fragment f of a step: f < TMI is the A fragment of tile row f, otherwise the B fragment f - TMI
+  auto load_frag_item = [&](int stage, int s, int f, Frag* fa, Frag* fb) {
+#ifdef KCG_DBG_NOFRAG
+    return;
+#endif
+    const int c = s * KH + fgrp;
+    if (f < TMI)
+      copy_bytes<16>(&fa[f], smA + stage * BM * CH + L::slot(wy * WM + f * MF + frow, c));
+    else
+      copy_bytes<16>(&fb[f - TMI], smB + stage * BN * CH + L::slot(wx * WN + (f - TMI) * MF + frow, c));
+  };
   auto mma_frag = [&](const Frag* fa, const Frag* fb) {
 #pragma unroll
     for (int i = 0; i < TMI; ++i)
@@ -611,44 +900,117 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
   };
 
   constexpr int SPW = NSS / LSU;   // fragment steps of one tile handled by this wave's split-U slice
-  auto compute_tile = [&](int stage) {
-    if constexpr (C::REGP) {
-      Frag fa[2][TMI], fb[2][TNI];
-      load_frag(stage, wz, fa[0], fb[0]);
-#pragma unroll
-      for (int s = 0; s < SPW; ++s) {
-        if (s + 1 < SPW) load_frag(stage, (s + 1) * LSU + wz, fa[(s + 1) & 1], fb[(s + 1) & 1]);
-        mma_frag(fa[s & 1], fb[s & 1]);
-      }
-    } else {
-      Frag fa[TMI], fb[TNI];
-#pragma unroll
-      for (int s = 0; s < SPW; ++s) {
-        load_frag(stage, s * LSU + wz, fa, fb);
-        mma_frag(fa, fb);
-      }
-    }
-  };
+  constexpr int NM = TMI * TNI;    // matrix-core groups per step
+  constexpr int NF = TMI + TNI;    // fragments per step
+  constexpr int MT = SPW * NM;     // matrix-core groups per K tile: the time line of the pipelined loop
+  constexpr bool PIPE_OK = MT >= 4;
+  constexpr int BAR = (SPW - 1) * NM + NM / 2;                 // group in front of which the barrier stands
+  constexpr int WEND = cmax(1, cmin(BAR, (MT * 3) / 8));       // LDS writes occupy groups [0, WEND)
+  constexpr int LEND = cmin(MT, cmax(WEND + 1, (MT * 3) / 4)); // global loads occupy groups [WEND, LEND)
+  constexpr int FSPAN = cmax(1, (NM * 3) / 4);                 // next-step fragment reads: first 3/4 of a step
+  constexpr int NSPAN = cmax(1, ((MT - BAR) * 3) / 4);         // next-tile fragment reads: behind the barrier
 
   // ---- K loop ---------------------------------------------------------------------------------
+  // SHARED_PREFETCH=1: two LDS stages, one barrier per K tile.  Registers carry tile kt+1 (fetched from
+  // global memory during tile kt-1); it is written to the idle stage at the start of tile kt, under
+  // the matrix-core work of that tile, and the fetch of tile kt+2 is issued right after.
+  // REG_PREFETCH=1 additionally keeps fragments one step ahead: the barrier sits before the last
+  // step's matrix-core work, and the first fragments of the next tile are read behind it, so their
+  // LDS latency is covered by that work.
   if constexpr (C::SHMP) {
     load_global(0);
     store_lds(0);
+    if (KT > 1) load_global(1);
     __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-      const int cur = kt & 1;
-      if (kt + 1 < KT) load_global(kt + 1);
-      compute_tile(cur);
-      if (kt + 1 < KT) store_lds(cur ^ 1);
-      __syncthreads();
+    if constexpr (C::REGP && PIPE_OK) {
+      // Software pipeline: the tile's MT = SPW*NM matrix-core groups are the time line; LDS writes of
+      // tile kt+1 go under the first groups, the global fetch of tile kt+2 under the following ones,
+      // fragment reads of step s+1 under step s; the barrier stands in the middle of the last step
+      // and the first fragments of tile kt+1 are read right behind it.  sched_barrier pins that order.
+      Frag fa[2][TMI], fb[2][TNI];
+      load_frag(0, wz, fa[0], fb[0]);
+      auto tile = [&](int kt, auto has1, auto has2) {
+        constexpr bool H1 = decltype(has1)::value, H2 = decltype(has2)::value;
+        const int cur = kt & 1;
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+#pragma unroll
+          for (int q = 0; q < NM; ++q) {
+            const int slot = s * NM + q;
+#ifndef KCG_DBG_NOBAR
+            if (slot == BAR) __syncthreads();
+#endif
+#ifndef KCG_DBG_NOMFMA
+            MI::run(acc[q / TNI][q % TNI], fa[s & 1][q / TNI], fb[s & 1][q % TNI]);
+#else
+            if (q == 0) { acc[0][0][0] += (float)fa[s & 1][0][0] + (float)fb[s & 1][0][0]; for (int ii = 1; ii < TMI; ++ii) acc[ii][0][0] += (float)fa[s & 1][ii][0] + (float)fb[s & 1][ii % TNI][0]; }
+#endif
+            if constexpr (H1) {
+#pragma unroll
+              for (int i = 0; i < NWR; ++i)
+                if ((i * WEND) / NWR == slot) write_item(i, cur ^ 1);
+            }
+            if constexpr (H2) {
+#pragma unroll
+              for (int i = 0; i < NLD; ++i)
+                if (WEND + (i * (LEND - WEND)) / NLD == slot) load_item(i, (kt + 2) * BK);
+            }
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+              if (s + 1 < SPW && (f * FSPAN) / NF == q)
+                load_frag_item(cur, (s + 1) * LSU + wz, f, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+              if (H1 && BAR + (f * NSPAN) / NF == slot) load_frag_item(cur ^ 1, wz, f, fa[SPW & 1], fb[SPW & 1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        if constexpr (SPW % 2 == 1) {   // odd step count: the prefetched fragments sit in slot 1
+#pragma unroll
+          for (int i = 0; i < TMI; ++i) fa[0][i] = fa[1][i];
+#pragma unroll
+          for (int j = 0; j < TNI; ++j) fb[0][j] = fb[1][j];
+        }
+      };
+      for (int kt = 0; kt + 2 < KT; ++kt) tile(kt, BoolC<true>(), BoolC<true>());
+      if (KT >= 2) tile(KT - 2, BoolC<true>(), BoolC<false>());
+      tile(KT - 1, BoolC<false>(), BoolC<false>());
+    } else {
+      for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) store_lds(cur ^ 1);
+        if (kt + 2 < KT) load_global(kt + 2);
+        Frag fa[TMI], fb[TNI];
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+          load_frag(cur, s * LSU + wz, fa, fb);
+          mma_frag(fa, fb);
+        }
+        __syncthreads();
+      }
     }
   } else {
+    // single LDS stage (the reference's unpipelined order, Optimizer.cc:343-376)
     for (int kt = 0; kt < KT; ++kt) {
       load_global(kt);
       __syncthreads();
       store_lds(0);
       __syncthreads();
-      compute_tile(0);
+      if constexpr (C::REGP) {
+        Frag fa[2][TMI], fb[2][TNI];
+        load_frag(0, wz, fa[0], fb[0]);
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+          if (s + 1 < SPW) load_frag(0, (s + 1) * LSU + wz, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+          mma_frag(fa[s & 1], fb[s & 1]);
+        }
+      } else {
+        Frag fa[TMI], fb[TNI];
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+          load_frag(0, s * LSU + wz, fa, fb);
+          mma_frag(fa, fb);
+        }
+      }
     }
   }
 

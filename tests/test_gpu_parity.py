@@ -82,6 +82,22 @@ HALF_CASES = [
     ("f16-edge", dict(M=200, N=136, K=100, dtype=2, dtype_c=4, is_atrans=0, BK=32)),
     ("f16-glw4", dict(M=256, N=256, K=128, dtype=2, dtype_c=4, is_atrans=1, BK=32, glw=4)),
     ("f16-out16", dict(M=256, N=256, K=128, dtype=2, is_atrans=0, BK=32)),
+    ("f16-direct-at1", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8, BK=64,
+                            shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-bk32", dict(M=256, N=384, K=224, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=32,
+                             shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-16x16", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=0, warp_layout=(4, 16), BM=64, BN=64,
+                              BK=32, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-16x16-at1", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=1, warp_layout=(16, 4), BM=64,
+                                  BN=64, BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-256", dict(M=512, N=512, K=512, dtype=2, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=16, TN=16, BK=64,
+                            shared_prefetch=1, reg_prefetch=1, block_mapping=4)),
+    ("f16-direct-256x128-8w", dict(M=512, N=512, K=192, dtype=2, dtype_c=4, is_atrans=1, BM=256, BN=128, TM=8, TN=8,
+                                   BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-direct", dict(M=256, N=256, K=256, dtype=3, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
+                         shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-out16", dict(M=256, N=256, K=128, dtype=2, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
+                              shared_prefetch=1, reg_prefetch=1)),
     ("bf16-at0", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=0, BK=32)),
     ("bf16-at1-lsu2", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=1, BK=64, lsu=2)),
 ]
