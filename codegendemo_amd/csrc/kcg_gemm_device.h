@@ -676,7 +676,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           __syncthreads();                                        // ... everyone's part; stage CUR is free
         }
         if (q == 0) wait_tr();   // fragments of this step (read under the previous step) are complete
-        MI::run(acc[q / TNI][q % TNI], fa[s & 1][q / TNI], fb[s & 1][q % TNI]);
+        // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
+        // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
+        MI::run(acc[q / TNI][q % TNI], fb[s & 1][q % TNI], fa[s & 1][q / TNI]);
         if constexpr (H2) {
 #pragma unroll
           for (int i = 0; i < NFETCH; ++i)
@@ -716,19 +718,24 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     tile(kt, No(), No(), No());
   }
 
-  // ---- epilogue (accumulator layout as in gemm_mfma) ---------------------------------------------
+  // ---- epilogue --------------------------------------------------------------------------------
+  // With swapped operands a 32x32 accumulator holds, per lane, row m = lane%32 and columns
+  // n = 8*g + 4*(lane/32) + {0..3} for g = 0..3 (16x16: row lane%16, columns 4*(lane/16) + {0..3}).
   constexpr int NACC = (int)(sizeof(Acc) / sizeof(float));
-  const int ocol = lane % MF;
-  const int orow = (lane / MF) * 4;
+  const int orow = lane % MF;
+  const int ocol = (lane / MF) * 4;
 #pragma unroll
   for (int i = 0; i < TMI; ++i)
 #pragma unroll
     for (int j = 0; j < TNI; ++j)
 #pragma unroll
-      for (int e = 0; e < NACC; ++e) {
-        const int row = m0 + wy * WM + i * MF + (e / 4) * 8 + orow + e % 4;
-        const int col = n0 + wx * WN + j * MF + ocol;
-        Cm[(long)row * N + col] = (TC)acc[i][j][e];
+      for (int g = 0; g < NACC / 4; ++g) {
+        const int row = m0 + wy * WM + i * MF + orow;
+        const int col = n0 + wx * WN + j * MF + g * 8 + ocol;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
+        gstore<TC, float, 4, false, true>(Cm, v, row, col, N, M, N);
       }
 }
 
@@ -802,12 +809,6 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
 
   auto load_item = [&](int idx, int k0) {
     int r, c;
-#ifdef KCG_DBG_SAMETILE
-    k0 = 0;
-#endif
-#ifdef KCG_DBG_NOLOAD
-    return;
-#endif
     if (idx < NLD_A) {
       const int it = idx / LPA, sub = idx % LPA;
       if constexpr (C::ATRANS) {   // r = k chunk, c = first m of the vector
@@ -824,9 +825,6 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
     }
   };
   auto write_item = [&](int idx, int stage) {
-#ifdef KCG_DBG_NOWRITE
-    return;
-#endif
     u32x4* sa = smA + stage * BM * CH;
     u32x4* sb = smB + stage * BN * CH;
     int r, c;
@@ -883,9 +881,6 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
   };
   // fragment f of a step: f < TMI is the A fragment of tile row f, otherwise the B fragment f - TMI
   auto load_frag_item = [&](int stage, int s, int f, Frag* fa, Frag* fb) {
-#ifdef KCG_DBG_NOFRAG
-    return;
-#endif
     const int c = s * KH + fgrp;
     if (f < TMI)
       copy_bytes<16>(&fa[f], smA + stage * BM * CH + L::slot(wy * WM + f * MF + frow, c));
@@ -937,14 +932,8 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
 #pragma unroll
           for (int q = 0; q < NM; ++q) {
             const int slot = s * NM + q;
-#ifndef KCG_DBG_NOBAR
             if (slot == BAR) __syncthreads();
-#endif
-#ifndef KCG_DBG_NOMFMA
             MI::run(acc[q / TNI][q % TNI], fa[s & 1][q / TNI], fb[s & 1][q % TNI]);
-#else
-            if (q == 0) { acc[0][0][0] += (float)fa[s & 1][0][0] + (float)fb[s & 1][0][0]; for (int ii = 1; ii < TMI; ++ii) acc[ii][0][0] += (float)fa[s & 1][ii][0] + (float)fb[s & 1][ii % TNI][0]; }
-#endif
             if constexpr (H1) {
 #pragma unroll
               for (int i = 0; i < NWR; ++i)

@@ -119,3 +119,25 @@ def make_config(M, N, K, BM=64, BN=64, BK=16, TM=4, TN=4, dtype=4, dtype_c=None,
         kw.KEY_UNROLL_NUM: unroll, kw.KEY_REG_PREFETCH: int(reg_prefetch), kw.KEY_SHARED_PREFETCH: int(shared_prefetch),
         kw.KEY_LOAD_CONTINUOUS: int(load_continuous), kw.KEY_REDUCE_C_CONTINUOUS: int(reduce_c_continuous),
     }
+
+
+def sweep_grid_points(param_options: dict):
+    """One config per point of the (BM, BN, BK, TM, TN, SHARED_PREFETCH, REG_PREFETCH) grid of a
+    tuning space: the first block/warp layout (in file order) that the engine accepts.  Returns
+    (configs, skipped) where skipped lists the grid points no layout can realise (e.g. a 32x32 tile
+    with 8x8 thread tiles has 16 threads, less than one wave) — skipped, not failed."""
+    kw = ConfigKeywords
+    grid_keys = [kw.KEY_BLOCK_SIZE_M, kw.KEY_BLOCK_SIZE_N, kw.KEY_BLOCK_SIZE_K, kw.KEY_THREAD_SIZE_M,
+                 kw.KEY_THREAD_SIZE_N, kw.KEY_SHARED_PREFETCH, kw.KEY_REG_PREFETCH]
+    seen, skipped = {}, []
+    opts = {k: (v if isinstance(v, (list, tuple)) else [v]) for k, v in param_options.items()}
+    for point in itertools.product(*[opts[k] for k in grid_keys]):
+        fixed = dict(opts)
+        for k, v in zip(grid_keys, point):
+            fixed[k] = [v]
+        first = next(iter_cfgs(fixed), None)
+        if first is None:
+            skipped.append(dict(zip(grid_keys, point)))
+        else:
+            seen[point] = first
+    return list(seen.values()), skipped
