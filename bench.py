@@ -29,6 +29,21 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6, "bf16": 2516.6}   # MI355X dense matrix peaks
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two passes), each scaled
+# by what the same counter read for a 256 MiB copy (FETCH x2.000, WRITE x1.000).  Keyed by the tile part
+# of the kernel name; a kernel that was not profiled reports null.
+MEASURED_TRAFFIC_BYTES = {
+    "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x16_BTmnk256x256x32_BLmn2x2": (2 * 196747 + 65536) * 1024,
+    "DTabcfloat16xfloat16xfloat32_AT0_TTmn16x16_BTmnk256x256x64_BLmn2x2": (2 * 98706 + 66048) * 1024,
+}
+
+
+def measured_traffic(kernel_name):
+    for key, nbytes in MEASURED_TRAFFIC_BYTES.items():
+        if key in kernel_name:
+            return nbytes
+    return None
+
 
 def load_tuned(name):
     path = name if os.path.isabs(name) or os.path.exists(name) else os.path.join(ROOT, "codegendemo_amd", "TunedConfigs", name)
@@ -130,6 +145,9 @@ def main():
     ap.add_argument("--no-fp16", action="store_true", help="skip the fp16 side measurement")
     ap.add_argument("--fp32-config", default="", help="JSON file ({'cfgs': [...]}) to use instead of the tuned fp32 config")
     ap.add_argument("--fp16-config", default="", help="same for the fp16 side measurement")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="profiling aid: first run a plain 256 MiB device copy three times, so that HBM counters "
+                         "(FETCH_SIZE / WRITE_SIZE) of the same profiler run can be scaled by a kernel of known traffic")
     ap.add_argument("--only-fp16", action="store_true",
                     help="profiling aid: run only the fp16 kernel (prints a reduced JSON line)")
     args = ap.parse_args()
@@ -144,6 +162,15 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0")     # 256 MiB
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     if args.only_fp16:
         cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
@@ -173,7 +200,7 @@ def main():
                    "kernel": info["kernel_name"], "kind": {1: "simt", 2: "mfma"}[info["kind"]],
                    "lds_bytes": info["lds_bytes"], "grid": info["grid"][0], "block": info["block"][0]},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS["f32"], "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_TFLOPS["f32"], "traffic": None,
+                     "frac": achieved / PEAK_TFLOPS["f32"], "traffic": measured_traffic(info["kernel_name"]),
                      "launch_ms": ms_launch,
                      "hbm_gbs_algorithmic": (4.0 * (kpm.M * kpm.K + kpm.K * kpm.N + kpm.M * kpm.N)) / (ms_launch * 1e-3) / 1e9},
     }
@@ -187,7 +214,8 @@ def main():
         out["fp16"] = {"value": flops / (ms_step16 * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_step16,
                        "dtype": "f16 in, f32 accumulate/out", "kernel": info16["kernel_name"],
                        "roofline": {"bound": "mfma", "achieved": ach16, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
-                                    "frac": ach16 / PEAK_TFLOPS["f16"], "launch_ms": ms_launch16}}
+                                    "frac": ach16 / PEAK_TFLOPS["f16"], "traffic": measured_traffic(info16["kernel_name"]),
+                                    "launch_ms": ms_launch16}}
 
     if not args.no_cpu:
         base, panel, rows = cpu_baseline(a, b)
