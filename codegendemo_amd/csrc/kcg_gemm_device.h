@@ -50,6 +50,15 @@ constexpr int cmin(int a, int b) { return a < b ? a : b; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 constexpr int lowbit(int a) { return a & (-a); }
 template <bool B> struct BoolC { static constexpr bool value = B; };
+template <int I> struct IntC { static constexpr int value = I; };
+// f(IntC<Begin>()), ..., f(IntC<End-1>()) — a loop whose index is a compile-time constant in the body
+template <int Begin, int End, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (Begin < End) {
+    f(IntC<Begin>());
+    static_for<Begin + 1, End>(f);
+  }
+}
 
 // Copy NBYTES (power of two, <= 16) between two suitably aligned addresses as one access.
 template <int NBYTES>
@@ -523,6 +532,10 @@ struct DirectPlan {
       SPW > 0 && SPW * NM >= 4 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
       (C::BM * C::BK / 8) % (64 * NW) == 0 && (C::BN * C::BK / 8) % (64 * NW) == 0 && (C::M % 8 == 0) &&
       (C::N % 8 == 0) && (C::K % 8 == 0) && 2 * (C::BM + C::BN) * C::BK * 2 <= 160 * 1024;
+  // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles)
+  static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * 2;
+  static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
+  static constexpr int NST = NST_FIT < 2 ? 2 : (NST_FIT > 4 ? 4 : NST_FIT);
   // the host picks the path (it must size dynamic LDS accordingly); both sides have to agree
   static_assert(ELIGIBLE == C::DIRECT, "host and device disagree on the direct-staging eligibility rule");
   static constexpr bool OK = C::DIRECT;
@@ -561,16 +574,26 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // The two stages are separate LDS objects on purpose: the compiler then knows that a fragment read
   // from one stage cannot alias an in-flight fetch into the other and does not wait for the fetch.
   // (For the same reason the K loop below is unrolled by two, so every access names its stage.)
+  constexpr int NST = P::NST;
   __shared__ __attribute__((aligned(1024))) char lds_stage0[STAGE_BYTES];
   __shared__ __attribute__((aligned(1024))) char lds_stage1[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char lds_stage2[NST > 2 ? STAGE_BYTES : 16];
+  __shared__ __attribute__((aligned(1024))) char lds_stage3[NST > 3 ? STAGE_BYTES : 16];
   (void)smem;
+  auto stage_ptr = [&](auto stage_c) -> char* {
+    constexpr int S = decltype(stage_c)::value;
+    if constexpr (S == 0) return lds_stage0;
+    else if constexpr (S == 1) return lds_stage1;
+    else if constexpr (S == 2) return lds_stage2;
+    else return lds_stage3;
+  };
 
   // swizzle of a row-contiguous tile: rows k..k+3 of a transposing read must not share banks
   auto swz_n = [](int k, int nch) { return ((k & 3) << 2) & (nch - 1); };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   auto fetch_item = [&](int idx, int kt, auto stage_c) {
-    char* st = decltype(stage_c)::value ? lds_stage1 : lds_stage0;
+    char* st = stage_ptr(stage_c);
     const int k0 = kt * BK;
     if (idx < NIA) {
       const int s = 64 * (wave * NIA + idx) + lane;   // physical chunk slot inside the A stage
@@ -606,7 +629,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // The transposing read is issued as inline assembly: as a builtin the compiler cannot tell that it
   // does not touch the stage a fetch is in flight to, and would drain all fetches (vmcnt(0)) in front
   // of every such read.  The price: the compiler does not know these reads are asynchronous either,
-  // so the loop below waits for them itself (wait_tr) before the matrix-core step that consumes them.
+  // so the loop below waits for them itself (wait_frags) before the matrix-core step that consumes them.
   auto read_tr = [&](const char* tile, int nch, int rowbase, int kb, Frag* dst) {
     const int n = rowbase + 16 * tsub + 4 * (tx % 4);
     u32x2 part[2];
@@ -618,10 +641,19 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     }
     copy_bytes<16>(dst, part);
   };
-  // lgkmcnt(0): every LDS read issued so far (compiler-visible or not) has returned
-  auto wait_tr = [&]() { __builtin_amdgcn_s_waitcnt(0xC07F); };
+  // lgkmcnt(0): every LDS read issued so far (compiler-visible or not) has returned.  The empty asm
+  // statements that follow make the fragments "outputs" of the wait, so the matrix-core instructions
+  // that consume them cannot be scheduled in front of it (volatile asm keeps its program order).
+  auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
+  auto wait_frags = [&](Frag* a, Frag* b) {
+    wait_lds();
+#pragma unroll
+    for (int i = 0; i < TMI; ++i) asm volatile("" : "+v"(a[i]));
+#pragma unroll
+    for (int j = 0; j < TNI; ++j) asm volatile("" : "+v"(b[j]));
+  };
   auto load_frag_item = [&](auto stage_c, int s, int f, Frag* fa, Frag* fb) {
-    const char* st = decltype(stage_c)::value ? lds_stage1 : lds_stage0;
+    const char* st = stage_ptr(stage_c);
     if (f < TMI) {
       if constexpr (AK) {
         const int row = wy * WM + f * MF + frow;
@@ -644,51 +676,73 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       for (int e = 0; e < (int)(sizeof(Acc) / sizeof(float)); ++e) acc[i][j][e] = 0.0f;
 
   // ---- K loop: two LDS stages; the barrier stands in the middle of the last step of a tile --------
+  // Schedule constants (time line = the MT matrix-core groups of a tile).  The defaults can be
+  // overridden per build with -DKCG_SCHED_...=n through $KCG_EXTRA_FLAGS when exploring schedules.
+#ifndef KCG_SCHED_BAR_Q
+#define KCG_SCHED_BAR_Q 0             /* barrier stands in front of this group of the last step */
+#endif
+#ifndef KCG_SCHED_FSPAN_PCT
+#define KCG_SCHED_FSPAN_PCT 50        /* next-step fragment reads are spread over this share of a step */
+#endif
+#ifndef KCG_SCHED_NSPAN_PCT
+#define KCG_SCHED_NSPAN_PCT 50        /* next-tile fragment reads: share of the groups behind the barrier */
+#endif
   constexpr int MT = SPW * NM;
-  constexpr int BAR = (SPW - 1) * NM + NM / 2;
-  constexpr int FSPAN = cmax(1, (NM * 3) / 4);
-  constexpr int NSPAN = cmax(1, ((MT - BAR) * 3) / 4);
+  constexpr int BAR = (SPW - 1) * NM + cmin(NM - 1, cmax(0, KCG_SCHED_BAR_Q));
+  constexpr int FSPAN = cmax(1, (NM * KCG_SCHED_FSPAN_PCT) / 100);
+  constexpr int NSPAN = cmax(1, ((MT - BAR) * KCG_SCHED_NSPAN_PCT) / 100);
   constexpr int TAIL = MT - BAR;
+  // s_waitcnt vmcnt(n), everything else unconstrained: n fetches of this wave may still be in flight
+  constexpr int VM_AHEAD = (NST - 2) * NFETCH;
+  static_assert(VM_AHEAD < 64, "vmcnt has 6 bits");
+  constexpr int WAIT_NEXT_TILE = 0x0F70 | (VM_AHEAD & 15) | ((VM_AHEAD >> 4) << 14);
 
+  // prologue: tile 0 -> stage 0, wait for it; then tiles 1..NST-1 in flight
 #pragma unroll
-  for (int i = 0; i < NFETCH; ++i) fetch_item(i, 0, BoolC<false>());
+  for (int i = 0; i < NFETCH; ++i) fetch_item(i, 0, IntC<0>());
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's chunks of tile 0 are in LDS
   __syncthreads();
-  if (KT > 1) {
+  static_for<1, NST>([&](auto t) {
+    if (decltype(t)::value < KT) {
 #pragma unroll
-    for (int i = 0; i < NFETCH; ++i) fetch_item(i, 1, BoolC<true>());
-  }
+      for (int i = 0; i < NFETCH; ++i) fetch_item(i, decltype(t)::value, t);
+    }
+  });
   Frag fa[2][TMI], fb[2][TNI];
 #pragma unroll
-  for (int f = 0; f < NF; ++f) load_frag_item(BoolC<false>(), 0, f, fa[0], fb[0]);
+  for (int f = 0; f < NF; ++f) load_frag_item(IntC<0>(), 0, f, fa[0], fb[0]);
 
-  // one K tile; `cur_c` is the stage it computes from, has1/has2: tiles kt+1 / kt+2 exist
-  auto tile = [&](int kt, auto cur_c, auto has1, auto has2) {
-    constexpr bool CUR = decltype(cur_c)::value;
-    constexpr bool H1 = decltype(has1)::value, H2 = decltype(has2)::value;
+  // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists (it is
+  // fetched into stage CUR as soon as the barrier of this tile has freed it).
+  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn) {
+    constexpr int CUR = decltype(cur_c)::value;
+    constexpr int NXT = (CUR + 1) % NST;
+    constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
 #pragma unroll
       for (int q = 0; q < NM; ++q) {
         const int slot = s * NM + q;
         if (slot == BAR) {
-          if constexpr (H1) __builtin_amdgcn_s_waitcnt(0x0F70);   // tile kt+1 has landed (this wave's part)
-          __syncthreads();                                        // ... everyone's part; stage CUR is free
+          // tile kt+1 has landed (this wave's part); tails of the K loop simply drain everything
+          if constexpr (H1) __builtin_amdgcn_s_waitcnt(HN ? WAIT_NEXT_TILE : 0x0F70);
+          wait_lds();        // this wave's reads of stage CUR have all returned (the compiler cannot see the asm ones)
+          __syncthreads();   // ... everyone's part; and every wave is done reading stage CUR
         }
-        if (q == 0) wait_tr();   // fragments of this step (read under the previous step) are complete
+        if (q == 0) wait_frags(fa[s & 1], fb[s & 1]);   // fragments of this step (read under the previous one) are complete
         // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
         // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
         MI::run(acc[q / TNI][q % TNI], fb[s & 1][q % TNI], fa[s & 1][q / TNI]);
-        if constexpr (H2) {
+        if constexpr (HN) {
 #pragma unroll
           for (int i = 0; i < NFETCH; ++i)
-            if (BAR + (i * TAIL) / NFETCH == slot) fetch_item(i, kt + 2, BoolC<CUR>());
+            if (BAR + (i * TAIL) / NFETCH == slot) fetch_item(i, kt + NST, IntC<CUR>());
         }
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
           if (s + 1 < SPW && (f * FSPAN) / NF == q)
-            load_frag_item(BoolC<CUR>(), s + 1, f, fa[(s + 1) & 1], fb[(s + 1) & 1]);
-          if (H1 && BAR + (f * NSPAN) / NF == slot) load_frag_item(BoolC<!CUR>(), 0, f, fa[SPW & 1], fb[SPW & 1]);
+            load_frag_item(IntC<CUR>(), s + 1, f, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+          if (H1 && BAR + (f * NSPAN) / NF == slot) load_frag_item(IntC<NXT>(), 0, f, fa[SPW & 1], fb[SPW & 1]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -700,23 +754,16 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       for (int j = 0; j < TNI; ++j) fb[0][j] = fb[1][j];
     }
   };
-  typedef BoolC<true> Yes;
-  typedef BoolC<false> No;
-  int kt = 0;
-  for (; kt + 3 < KT; kt += 2) {
-    tile(kt, No(), Yes(), Yes());
-    tile(kt + 1, Yes(), Yes(), Yes());
+  // main part: groups of NST tiles, every tile with both successors; the rest is unrolled with the
+  // right flags at compile time (KT is a constant)
+  constexpr int NG = (KT >= 2 * NST) ? (KT - 2 * NST) / NST + 1 : 0;
+  for (int g = 0; g < NG; ++g) {
+    static_for<0, NST>([&](auto sc) { tile(g * NST + decltype(sc)::value, sc, BoolC<true>(), BoolC<true>()); });
   }
-  if (KT - kt == 3) {
-    tile(kt, No(), Yes(), Yes());
-    tile(kt + 1, Yes(), Yes(), No());
-    tile(kt + 2, No(), No(), No());
-  } else if (KT - kt == 2) {
-    tile(kt, No(), Yes(), No());
-    tile(kt + 1, Yes(), No(), No());
-  } else {
-    tile(kt, No(), No(), No());
-  }
+  static_for<NG * NST, KT>([&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+    tile(T, IntC<T % NST>(), BoolC<(T + 1 < KT)>(), BoolC<(T + NST < KT)>());
+  });
 
   // ---- epilogue --------------------------------------------------------------------------------
   // With swapped operands a 32x32 accumulator holds, per lane, row m = lane%32 and columns
