@@ -1,0 +1,233 @@
+// kcg_runner — stand-alone (no Python) runner for the engine's GEMM kernels on one GPU.
+//
+// It plays the role of the reference's C++ check programs: runkernel.cpp (load a code object given on
+// the command line, launch it several times, compare against a naive GPU kernel with an absolute
+// tolerance of 0.01, runkernel.cpp:49-112) and the main() of matmul.cpp (HIP-event timing, TFLOPS
+// print, naive `gemm_kernel` + `verify_kernel`, matmul.cpp:2327-2348,2386-2553).
+//
+//   kcg_runner --config <file.json> [--index i] [--kind auto|simt|mfma] [--iters n] [--tol t]
+//       compiles entry i of a {"cfgs": [...]} file (or a single flat config object) through
+//       libkcg_gemm.so, loads it, verifies it against the naive kernel and times it
+//       (--compile-only 1 stops after the compile: fills the code-object cache on a host without a GPU)
+//   kcg_runner M N K gridX blockX <code-object> <kernel-name> [ldsBytes] [dtypeCode] [isATrans]
+//       the reference runner's argument list (runkernel.cpp:63-66): launches an existing code object
+//
+// Build: make -C codegendemo_amd/csrc runner      (hipcc --offload-arch=gfx950)
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/kcg_gemm.h"
+
+#define HIP_OK(x)                                                                      \
+  do {                                                                                 \
+    hipError_t e_ = (x);                                                               \
+    if (e_ != hipSuccess) {                                                            \
+      fprintf(stderr, "HIP error %d (%s) at %s:%d\n", (int)e_, hipGetErrorString(e_), __FILE__, __LINE__); \
+      exit(3);                                                                         \
+    }                                                                                  \
+  } while (0)
+
+// ---- naive reference kernel: one thread per C element, fp32 accumulation in ascending k -------------
+// (gemm_kernel, matmul.cpp:2327-2337, for both A layouts and any input type)
+template <class T>
+__global__ void gemm_naive(const T* __restrict__ A, const T* __restrict__ B, float* __restrict__ D, int M, int N, int K,
+                           int a_trans) {
+  const int col = blockIdx.x * blockDim.x + threadIdx.x;
+  const int row = blockIdx.y * blockDim.y + threadIdx.y;
+  if (row >= M || col >= N) return;
+  float acc = 0.f;
+  for (int k = 0; k < K; ++k) {
+    const float a = a_trans ? (float)A[(size_t)k * M + row] : (float)A[(size_t)row * K + k];
+    acc += a * (float)B[(size_t)k * N + col];
+  }
+  D[(size_t)row * N + col] = acc;
+}
+
+// ---- compare kernel: counts |C - D| >= tol (NaN counts), keeps the largest error and the first offender
+// (verify_kernel, matmul.cpp:2339-2348 printed offenders from the device; here they are counted)
+template <class TC>
+__global__ void verify(const TC* __restrict__ C, const float* __restrict__ D, size_t n, float tol,
+                       unsigned long long* bad, unsigned int* max_err_bits, unsigned long long* first_bad) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float err = fabsf((float)C[i] - D[i]);
+  if (!(err < tol)) {
+    atomicAdd(bad, 1ull);
+    atomicMin(first_bad, (unsigned long long)i);
+  }
+  if (err == err) atomicMax(max_err_bits, __float_as_uint(err));
+}
+
+static float lcg_uniform(uint64_t& s) {   // [-1, 1)
+  s = s * 6364136223846793005ull + 1442695040888963407ull;
+  return (float)((int32_t)(s >> 40) - (1 << 23)) / (float)(1 << 23);
+}
+
+template <class T>
+static void* upload(const std::vector<float>& h) {
+  std::vector<T> t(h.size());
+  for (size_t i = 0; i < h.size(); ++i) t[i] = (T)h[i];
+  void* d;
+  HIP_OK(hipMalloc(&d, t.size() * sizeof(T)));
+  HIP_OK(hipMemcpy(d, t.data(), t.size() * sizeof(T), hipMemcpyHostToDevice));
+  return d;
+}
+
+// minimal reader for the flat {"KEY": int, ...} objects of the tuning files
+static bool read_config(const std::string& path, int index, kcg_matmul_cfg* cfg) {
+  std::ifstream f(path);
+  if (!f) return false;
+  std::stringstream ss;
+  ss << f.rdbuf();
+  std::string text = ss.str();
+  size_t start = 0;
+  size_t arr = text.find("\"cfgs\"");
+  if (arr != std::string::npos) {
+    start = text.find('[', arr);
+    for (int i = 0; i <= index; ++i) {
+      start = text.find('{', start + (i ? 1 : 0));
+      if (start == std::string::npos) return false;
+      if (i < index) start = text.find('}', start);
+    }
+  }
+  size_t end = text.find('}', start);
+  std::string obj = text.substr(start, end - start);
+  for (int i = 0; i < KCG_CFG_LEN; ++i) {
+    std::string key = std::string("\"") + kcg_cfg_keyword(i) + "\"";
+    size_t p = obj.find(key);
+    if (p == std::string::npos) {
+      fprintf(stderr, "config is missing %s\n", key.c_str());
+      return false;
+    }
+    p = obj.find(':', p);
+    cfg->v[i] = (int32_t)strtol(obj.c_str() + p + 1, nullptr, 10);
+  }
+  return true;
+}
+
+int main(int argc, char** argv) {
+  kcg_matmul_cfg cfg;
+  memset(&cfg, 0, sizeof(cfg));
+  kcg_kernel_info info;
+  memset(&info, 0, sizeof(info));
+  int iters = 20, kind = KCG_KIND_AUTO, index = 0, compile_only = 0;
+  float tol = 0.01f;   // the reference runner's tolerance (runkernel.cpp:34)
+  int M = 0, N = 0, K = 0, dt = KCG_DT_FLOAT32, dtc = KCG_DT_FLOAT32, atrans = 1;
+
+  if (argc >= 3 && !strcmp(argv[1], "--config")) {
+    std::string path = argv[2];
+    for (int i = 3; i + 1 < argc; i += 2) {
+      if (!strcmp(argv[i], "--index")) index = atoi(argv[i + 1]);
+      else if (!strcmp(argv[i], "--iters")) iters = atoi(argv[i + 1]);
+      else if (!strcmp(argv[i], "--tol")) tol = (float)atof(argv[i + 1]);
+      else if (!strcmp(argv[i], "--compile-only")) compile_only = atoi(argv[i + 1]);
+      else if (!strcmp(argv[i], "--kind"))
+        kind = !strcmp(argv[i + 1], "simt") ? KCG_KIND_SIMT : !strcmp(argv[i + 1], "mfma") ? KCG_KIND_MFMA : KCG_KIND_AUTO;
+    }
+    if (!read_config(path, index, &cfg)) {
+      fprintf(stderr, "cannot read config %d of %s\n", index, path.c_str());
+      return 2;
+    }
+    if (kcg_compile_matmul(&cfg, "gfx950", kind, &info) != KCG_OK) {
+      fprintf(stderr, "compile failed: %s\n", kcg_last_error());
+      return 2;
+    }
+    M = cfg.v[KCG_M]; N = cfg.v[KCG_N]; K = cfg.v[KCG_K];
+    dt = cfg.v[KCG_DTYPE_A]; dtc = cfg.v[KCG_DTYPE_C]; atrans = cfg.v[KCG_IS_ATRANS];
+    printf("compiled %s (%s kernel, cache %s)\n", info.kernel_name, info.kind == KCG_KIND_MFMA ? "matrix-core" : "SIMT",
+           info.cache_hit ? "hit" : "miss");
+    if (compile_only) return 0;
+  } else if (argc >= 8) {
+    M = atoi(argv[1]); N = atoi(argv[2]); K = atoi(argv[3]);
+    info.grid[0] = atoi(argv[4]); info.grid[1] = info.grid[2] = 1;
+    info.block[0] = atoi(argv[5]); info.block[1] = info.block[2] = 1;
+    snprintf(info.code_path, sizeof(info.code_path), "%s", argv[6]);
+    snprintf(info.kernel_name, sizeof(info.kernel_name), "%s", argv[7]);
+    info.lds_bytes = argc > 8 ? atoi(argv[8]) : 2048;   // runkernel.cpp launched with 2048 B of dynamic LDS
+    if (argc > 9) dt = atoi(argv[9]);
+    dtc = (dt == KCG_DT_FLOAT64) ? dt : KCG_DT_FLOAT32;
+    if (argc > 10) atrans = atoi(argv[10]);
+    iters = 7;                                           // runkernel.cpp:104-108
+  } else {
+    fprintf(stderr, "usage: %s --config file.json [--index i] [--kind auto|simt|mfma] [--iters n] [--tol t] [--compile-only 1]\n"
+                    "       %s M N K gridX blockX code-object kernel-name [ldsBytes] [dtypeCode] [isATrans]\n", argv[0], argv[0]);
+    return 2;
+  }
+  if (dt == KCG_DT_FLOAT64 || (dtc != KCG_DT_FLOAT32)) {
+    fprintf(stderr, "runner verifies float32-output kernels with float32/float16/bfloat16 inputs\n");
+    return 2;
+  }
+
+  // inputs: logical A[M,K], laid out as the kernel expects
+  uint64_t seed = 0x4B4347;
+  std::vector<float> a((size_t)M * K), b((size_t)K * N), abuf((size_t)M * K);
+  for (auto& x : a) x = lcg_uniform(seed);
+  for (auto& x : b) x = lcg_uniform(seed);
+  if (atrans) {
+    for (int i = 0; i < M; ++i)
+      for (int k = 0; k < K; ++k) abuf[(size_t)k * M + i] = a[(size_t)i * K + k];
+  } else {
+    abuf = a;
+  }
+  void *dA, *dB;
+  float *dC, *dD;
+  if (dt == KCG_DT_FLOAT32) { dA = upload<float>(abuf); dB = upload<float>(b); }
+  else if (dt == KCG_DT_FLOAT16) { dA = upload<_Float16>(abuf); dB = upload<_Float16>(b); }
+  else { dA = upload<__bf16>(abuf); dB = upload<__bf16>(b); }
+  HIP_OK(hipMalloc(&dC, (size_t)M * N * sizeof(float)));
+  HIP_OK(hipMalloc(&dD, (size_t)M * N * sizeof(float)));
+  HIP_OK(hipMemset(dC, 0xFF, (size_t)M * N * sizeof(float)));   // NaN pattern: unwritten elements fail the check
+
+  uint64_t module = 0, function = 0;
+  int32_t regs = 0, spills = 0;
+  if (kcg_load(info.code_path, info.kernel_name, info.lds_bytes, 0, &module, &function, &regs, &spills) != KCG_OK) {
+    fprintf(stderr, "load failed: %s\n", kcg_last_error());
+    return 3;
+  }
+  printf("M=%d N=%d K=%d grid=%d block=%d lds=%d B regs=%d scratch=%d dwords\n", M, N, K, info.grid[0], info.block[0],
+         info.lds_bytes, regs, spills);
+
+  if (kcg_launch(function, info.grid, info.block, info.lds_bytes, 0, (uint64_t)dA, (uint64_t)dB, (uint64_t)dC) != KCG_OK) {
+    fprintf(stderr, "launch failed: %s\n", kcg_last_error());
+    return 3;
+  }
+  dim3 nb(16, 16), ng((N + 15) / 16, (M + 15) / 16);
+  if (dt == KCG_DT_FLOAT32) hipLaunchKernelGGL(gemm_naive<float>, ng, nb, 0, 0, (const float*)dA, (const float*)dB, dD, M, N, K, atrans);
+  else if (dt == KCG_DT_FLOAT16) hipLaunchKernelGGL(gemm_naive<_Float16>, ng, nb, 0, 0, (const _Float16*)dA, (const _Float16*)dB, dD, M, N, K, atrans);
+  else hipLaunchKernelGGL(gemm_naive<__bf16>, ng, nb, 0, 0, (const __bf16*)dA, (const __bf16*)dB, dD, M, N, K, atrans);
+  unsigned long long *dBad, *dFirst;
+  unsigned int* dMax;
+  HIP_OK(hipMalloc(&dBad, 8)); HIP_OK(hipMalloc(&dFirst, 8)); HIP_OK(hipMalloc(&dMax, 4));
+  HIP_OK(hipMemset(dBad, 0, 8)); HIP_OK(hipMemset(dFirst, 0xFF, 8)); HIP_OK(hipMemset(dMax, 0, 4));
+  const size_t n = (size_t)M * N;
+  hipLaunchKernelGGL(verify<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0, dC, dD, n, tol, dBad, dMax, dFirst);
+  HIP_OK(hipDeviceSynchronize());
+  unsigned long long bad = 0, first = 0;
+  unsigned int maxbits = 0;
+  HIP_OK(hipMemcpy(&bad, dBad, 8, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(&first, dFirst, 8, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(&maxbits, dMax, 4, hipMemcpyDeviceToHost));
+  float maxerr;
+  memcpy(&maxerr, &maxbits, 4);
+  if (bad) printf("have %llu error! first at (y=%llu, x=%llu), max |err| %.3e (tol %.3g)\n", bad, first / N, first % N, maxerr, tol);
+  else printf("no error! max |err| %.3e (tol %.3g)\n", maxerr, tol);
+
+  float med = 0.f, mn = 0.f;
+  if (kcg_benchmark(function, info.grid, info.block, info.lds_bytes, 0, (uint64_t)dA, (uint64_t)dB, (uint64_t)dC, 20, iters, 0,
+                    &med, &mn) != KCG_OK) {
+    fprintf(stderr, "benchmark failed: %s\n", kcg_last_error());
+    return 3;
+  }
+  printf("time cost: %.4f ms (median of %d), min %.4f ms;  tflops = %.2f\n", med, iters, mn,
+         2.0 * M * N * K / (med * 1e-3) / 1e12);
+  kcg_unload(module);
+  return bad ? 1 : 0;
+}

@@ -1,0 +1,60 @@
+"""The stand-alone C++ runner (naive device GEMM + compare kernel + event timing), both argument forms:
+the twin of the reference's runkernel.cpp / matmul.cpp main programs."""
+import json
+import os
+import subprocess
+
+import pytest
+
+from codegendemo_amd import _native
+from codegendemo_amd.kcg.ConfigGenerator import make_config
+from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
+
+pytestmark = pytest.mark.gpu
+
+RUNNER = os.path.join(os.path.dirname(_native.LIB_PATH), "kcg_runner")
+
+CASES = {
+    "f32-mfma": (make_config(1024, 1024, 1024, BM=64, BN=64, BK=16, TM=4, TN=4, is_atrans=0), "mfma"),
+    "f32-simt-at": (make_config(1024, 1024, 1024, BM=64, BN=64, BK=16, TM=4, TN=4, is_atrans=1), "simt"),
+    "f16-direct": (make_config(1024, 1024, 1024, dtype=2, dtype_c=4, BM=128, BN=128, BK=64, TM=8, TN=8, is_atrans=0,
+                               shared_prefetch=1, reg_prefetch=1), "auto"),
+}
+
+
+def _run(args):
+    assert os.path.exists(RUNNER), "kcg_runner is not built (make -C codegendemo_amd/csrc runner)"
+    p = subprocess.run([RUNNER] + [str(a) for a in args], capture_output=True, text=True, timeout=120)
+    print(p.stdout, p.stderr, flush=True)
+    return p
+
+
+@pytest.mark.parametrize("case", list(CASES))
+def test_runner_config_mode(case, tmp_path):
+    cfg, kind = CASES[case]
+    path = tmp_path / "cfg.json"
+    path.write_text(json.dumps({"cfgs": [make_config(256, 256, 256, BM=64, BN=64, BK=16, TM=4, TN=4), cfg]}))
+    print(f"[case] kcg_runner --config {case}", flush=True)
+    p = _run(["--config", path, "--index", 1, "--kind", kind, "--iters", 5])
+    assert p.returncode == 0
+    assert "no error!" in p.stdout and "tflops" in p.stdout
+
+
+def test_runner_reference_argument_list():
+    """M N K gridX blockX code-object kernel-name ldsBytes dtype isATrans — runkernel.cpp's contract."""
+    cfg, _ = CASES["f32-mfma"]
+    info = _native.compile_matmul(kernelArgFromConfig(cfg).values(), "gfx950", _native.KIND_MFMA)
+    print("[case] kcg_runner positional", flush=True)
+    p = _run([1024, 1024, 1024, info["grid"][0], info["block"][0], info["code_path"], info["kernel_name"],
+              info["lds_bytes"], 4, 0])
+    assert p.returncode == 0 and "no error!" in p.stdout
+
+
+def test_runner_reports_a_wrong_kernel():
+    """Launched with A declared transposed although the kernel reads it row-major, the compare kernel
+    must count errors and the exit status must say so (every access stays in bounds: M == K)."""
+    cfg, _ = CASES["f32-mfma"]
+    info = _native.compile_matmul(kernelArgFromConfig(cfg).values(), "gfx950", _native.KIND_MFMA)
+    p = _run([1024, 1024, 1024, info["grid"][0], info["block"][0], info["code_path"], info["kernel_name"],
+              info["lds_bytes"], 4, 1])
+    assert p.returncode == 1 and "error!" in p.stdout and "no error!" not in p.stdout
