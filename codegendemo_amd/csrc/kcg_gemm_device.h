@@ -50,6 +50,8 @@ constexpr int cmin(int a, int b) { return a < b ? a : b; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 constexpr int lowbit(int a) { return a & (-a); }
 template <bool B> struct BoolC { static constexpr bool value = B; };
+template <bool B, class X, class Y> struct Select { typedef X type; };
+template <class X, class Y> struct Select<false, X, Y> { typedef Y type; };
 template <int I> struct IntC { static constexpr int value = I; };
 // f(IntC<Begin>()), ..., f(IntC<End-1>()) — a loop whose index is a compile-time constant in the body
 template <int Begin, int End, class F>
@@ -565,13 +567,15 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   typedef LdsTile<CHK> LK;
 
   const int tid = threadIdx.x;
-  const int wave = tid / 64, lane = tid % 64;
+  // the wave number is the same in all lanes: saying so keeps everything derived from it (LDS fetch
+  // destinations, which go through M0, and the wave's tile origin) in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
   const int wy = wave / C::BLN, wx = wave % C::BLN;
   int by, bx;
   block_coords<C>(blockIdx.x, by, bx);
   const int m0 = by * BM, n0 = bx * BN;
 
-  // The two stages are separate LDS objects on purpose: the compiler then knows that a fragment read
+  // The stages are separate LDS objects on purpose: the compiler then knows that a fragment read
   // from one stage cannot alias an in-flight fetch into the other and does not wait for the fetch.
   // (For the same reason the K loop below is unrolled by two, so every access names its stage.)
   constexpr int NST = P::NST;
@@ -592,29 +596,55 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   auto swz_n = [](int k, int nch) { return ((k & 3) << 2) & (nch - 1); };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------
-  auto fetch_item = [&](int idx, int kt, auto stage_c) {
+  // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
+  // never changes: the K loop spends no vector instruction on addresses.
+  static_assert((long)BM * K * 2 < (1L << 31) && (long)BK * M * 2 < (1L << 31) && (long)BK * N * 2 < (1L << 31),
+                "32-bit lane offsets");
+  unsigned voff_a[NIA], voff_b[NIB];
+#pragma unroll
+  for (int idx = 0; idx < NIA; ++idx) {
+    const int s = 64 * (wave * NIA + idx) + lane;     // physical chunk slot inside the A stage
+    if constexpr (AK) {
+      const int row = s / CHK, cp = s % CHK;
+      const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
+      voff_a[idx] = (unsigned)((row * K + c * 8) * 2);
+    } else {
+      const int k = s / NCHA, cp = s % NCHA;
+      const int c = cp ^ swz_n(k, NCHA);
+      voff_a[idx] = (unsigned)((k * M + c * 8) * 2);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) {
+    const int s = 64 * (wave * NIB + j) + lane;
+    const int k = s / NCHB, cp = s % NCHB;
+    const int c = cp ^ swz_n(k, NCHB);
+    voff_b[j] = (unsigned)((k * N + c * 8) * 2);
+  }
+  const char* const a_base = (const char*)(AK ? A + (long)m0 * K : A + m0);
+  const char* const b_base = (const char*)(B + n0);
+  constexpr long A_KT_BYTES = AK ? (long)BK * 2 : (long)BK * M * 2;   // one K tile further
+  constexpr long B_KT_BYTES = (long)BK * N * 2;
+  // The tile bases pass through an empty asm: the compiler must not fold the per-tile scalar part
+  // into the per-lane part (it would hoist "base + lane offset" as a 64-bit vector value and add the
+  // tile offset with vector instructions); kept apart, the fetch uses its scalar-base addressing form.
+  struct TileBase { const char* a; const char* b; };
+  auto tile_base = [&](int kt) {
+    TileBase t = {a_base + kt * A_KT_BYTES, b_base + kt * B_KT_BYTES};
+    asm("" : "+s"(t.a), "+s"(t.b));
+    return t;
+  };
+  auto fetch_item = [&](int idx, const TileBase& tb, auto stage_c) {
     char* st = stage_ptr(stage_c);
-    const int k0 = kt * BK;
     if (idx < NIA) {
-      const int s = 64 * (wave * NIA + idx) + lane;   // physical chunk slot inside the A stage
-      const T* src;
-      if constexpr (AK) {
-        const int row = s / CHK, cp = s % CHK;
-        const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
-        src = A + (long)(m0 + row) * K + k0 + c * 8;
-      } else {
-        const int k = s / NCHA, cp = s % NCHA;
-        const int c = cp ^ swz_n(k, NCHA);
-        src = A + (long)(k0 + k) * M + m0 + c * 8;
-      }
+      asm volatile("" : "+v"(voff_a[idx]));   // keeps the 32->64 bit extension next to the fetch (see tile_base)
+      const char* src = tb.a + (unsigned long)voff_a[idx];
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(st + 1024 * (wave * NIA + idx)), 16, 0, 0);
     } else {
       const int j = idx - NIA;
-      const int s = 64 * (wave * NIB + j) + lane;
-      const int k = s / NCHB, cp = s % NCHB;
-      const int c = cp ^ swz_n(k, NCHB);
-      const T* src = B + (long)(k0 + k) * N + n0 + c * 8;
+      asm volatile("" : "+v"(voff_b[j]));
+      const char* src = tb.b + (unsigned long)voff_b[j];
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(st + A_BYTES + 1024 * (wave * NIB + j)), 16, 0, 0);
     }
@@ -630,34 +660,51 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // does not touch the stage a fetch is in flight to, and would drain all fetches (vmcnt(0)) in front
   // of every such read.  The price: the compiler does not know these reads are asynchronous either,
   // so the loop below waits for them itself (wait_frags) before the matrix-core step that consumes them.
-  auto read_tr = [&](const char* tile, int nch, int rowbase, int kb, Frag* dst) {
+  // A fragment read with the transposing instruction lives in two 64-bit halves until the matrix-core
+  // instruction that consumes it: those reads are asynchronous and invisible to the compiler, so
+  // their destination registers must stay the asm outputs themselves (never a copy made before the
+  // data has arrived).  Fragments read with an ordinary 128-bit load are one value.
+  struct FragTr {
+    u32x2 h[2];
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
+    __device__ __forceinline__ Frag get() const {
+      const u32x4 v = {h[0].x, h[0].y, h[1].x, h[1].y};
+      return __builtin_bit_cast(Frag, v);
+    }
+  };
+  struct FragLd {
+    u32x4 q;
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(q)); }
+    __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
+  };
+  typedef typename Select<AK, FragLd, FragTr>::type FragA;
+  typedef FragTr FragB;
+  auto read_tr = [&](const char* tile, int nch, int rowbase, int kb, FragTr* dst) {
     const int n = rowbase + 16 * tsub + 4 * (tx % 4);
-    u32x2 part[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int k = kb + 4 * t + tx / 4;
       const unsigned addr = (unsigned)(unsigned long)(tile + ((k * nch + ((n / 8) ^ swz_n(k, nch))) * 16) + (n % 8) * 2);
-      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(part[t]) : "v"(addr));
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst->h[t]) : "v"(addr));
     }
-    copy_bytes<16>(dst, part);
   };
   // lgkmcnt(0): every LDS read issued so far (compiler-visible or not) has returned.  The empty asm
   // statements that follow make the fragments "outputs" of the wait, so the matrix-core instructions
   // that consume them cannot be scheduled in front of it (volatile asm keeps its program order).
   auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
-  auto wait_frags = [&](Frag* a, Frag* b) {
+  auto wait_frags = [&](FragA* a, FragB* b) {
     wait_lds();
 #pragma unroll
-    for (int i = 0; i < TMI; ++i) asm volatile("" : "+v"(a[i]));
+    for (int i = 0; i < TMI; ++i) a[i].pin();
 #pragma unroll
-    for (int j = 0; j < TNI; ++j) asm volatile("" : "+v"(b[j]));
+    for (int j = 0; j < TNI; ++j) b[j].pin();
   };
-  auto load_frag_item = [&](auto stage_c, int s, int f, Frag* fa, Frag* fb) {
+  auto load_frag_item = [&](auto stage_c, int s, int f, FragA* fa, FragB* fb) {
     const char* st = stage_ptr(stage_c);
     if (f < TMI) {
       if constexpr (AK) {
         const int row = wy * WM + f * MF + frow;
-        copy_bytes<16>(&fa[f], st + LK::slot(row, s * KH + fgrp) * 16);
+        fa[f].q = *(const u32x4*)(st + LK::slot(row, s * KH + fgrp) * 16);
       } else {
         read_tr(st, NCHA, wy * WM + f * MF, s * KS + 8 * fgrp, &fa[f]);
       }
@@ -699,16 +746,17 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 
   // prologue: tile 0 -> stage 0, wait for it; then tiles 1..NST-1 in flight
 #pragma unroll
-  for (int i = 0; i < NFETCH; ++i) fetch_item(i, 0, IntC<0>());
+  for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(0), IntC<0>());
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's chunks of tile 0 are in LDS
   __syncthreads();
   static_for<1, NST>([&](auto t) {
     if (decltype(t)::value < KT) {
 #pragma unroll
-      for (int i = 0; i < NFETCH; ++i) fetch_item(i, decltype(t)::value, t);
+      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t);
     }
   });
-  Frag fa[2][TMI], fb[2][TNI];
+  FragA fa[2][TMI];
+  FragB fb[2][TNI];
 #pragma unroll
   for (int f = 0; f < NF; ++f) load_frag_item(IntC<0>(), 0, f, fa[0], fb[0]);
 
@@ -718,6 +766,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     constexpr int CUR = decltype(cur_c)::value;
     constexpr int NXT = (CUR + 1) % NST;
     constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
+    const TileBase tbn = tile_base(HN ? kt + NST : 0);
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
 #pragma unroll
@@ -732,11 +781,11 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         if (q == 0) wait_frags(fa[s & 1], fb[s & 1]);   // fragments of this step (read under the previous one) are complete
         // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
         // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
-        MI::run(acc[q / TNI][q % TNI], fb[s & 1][q % TNI], fa[s & 1][q / TNI]);
+        MI::run(acc[q / TNI][q % TNI], fb[s & 1][q % TNI].get(), fa[s & 1][q / TNI].get());
         if constexpr (HN) {
 #pragma unroll
           for (int i = 0; i < NFETCH; ++i)
-            if (BAR + (i * TAIL) / NFETCH == slot) fetch_item(i, kt + NST, IntC<CUR>());
+            if (BAR + (i * TAIL) / NFETCH == slot) fetch_item(i, tbn, IntC<CUR>());
         }
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
