@@ -722,7 +722,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 #pragma unroll
       for (int e = 0; e < (int)(sizeof(Acc) / sizeof(float)); ++e) acc[i][j][e] = 0.0f;
 
-  // ---- K loop: two LDS stages; the barrier stands in the middle of the last step of a tile --------
+  // ---- K loop: NST LDS stages; the barrier stands in front of the last step of a tile -----------------
   // Schedule constants (time line = the MT matrix-core groups of a tile).  The defaults can be
   // overridden per build with -DKCG_SCHED_...=n through $KCG_EXTRA_FLAGS when exploring schedules.
 #ifndef KCG_SCHED_BAR_Q
@@ -740,9 +740,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int NSPAN = cmax(1, ((MT - BAR) * KCG_SCHED_NSPAN_PCT) / 100);
   constexpr int TAIL = MT - BAR;
   // s_waitcnt vmcnt(n), everything else unconstrained: n fetches of this wave may still be in flight
-  constexpr int VM_AHEAD = (NST - 2) * NFETCH;
-  static_assert(VM_AHEAD < 64, "vmcnt has 6 bits");
-  constexpr int WAIT_NEXT_TILE = 0x0F70 | (VM_AHEAD & 15) | ((VM_AHEAD >> 4) << 14);
+  static_assert((NST - 2) * NFETCH < 64, "vmcnt has 6 bits");
+  auto vmcnt_only = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
+  auto tiles_ahead = [](int t) {
+    const int last = cmin(KT - 1, cmax(t, 1) - 1 + NST);
+    return cmax(0, last - (t + 1));
+  };
 
   // prologue: tile 0 -> stage 0, wait for it; then tiles 1..NST-1 in flight
 #pragma unroll
@@ -760,32 +763,49 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 #pragma unroll
   for (int f = 0; f < NF; ++f) load_frag_item(IntC<0>(), 0, f, fa[0], fb[0]);
 
-  // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists (it is
-  // fetched into stage CUR as soon as the barrier of this tile has freed it).
-  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn) {
+  // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists; HP: the
+  // fetch of tile kt-1+NST, begun behind the previous tile's barrier, is still being issued.
+  //
+  // A stage is free once the barrier of the tile that computed from it has been passed, and the tile
+  // fetched into it is needed NST-1 barriers later.  With three or more stages its NFETCH fetch
+  // instructions are spread over the whole period up to the next barrier (the memory pipeline of a CU
+  // takes 16 cycles per 1 KiB fetch instruction; four waves issuing all of theirs right behind the
+  // barrier would stall on it); with two stages they must all be issued in the rest of this tile.
+  constexpr int SPREAD = NST >= 3 ? MT : TAIL;
+  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c) {
     constexpr int CUR = decltype(cur_c)::value;
-    constexpr int NXT = (CUR + 1) % NST;
+    constexpr int NXT = (CUR + 1) % NST, PRV = (CUR + NST - 1) % NST;
     constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
+    constexpr bool HP = decltype(hasp)::value && SPREAD > TAIL;
     const TileBase tbn = tile_base(HN ? kt + NST : 0);
+    const TileBase tbp = tile_base(HP ? kt - 1 + NST : 0);
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
 #pragma unroll
       for (int q = 0; q < NM; ++q) {
         const int slot = s * NM + q;
         if (slot == BAR) {
-          // tile kt+1 has landed (this wave's part); tails of the K loop simply drain everything
-          if constexpr (H1) __builtin_amdgcn_s_waitcnt(HN ? WAIT_NEXT_TILE : 0x0F70);
+          // tile kt+1 has landed (this wave's part): of the fetches issued so far only those of the
+          // tiles behind it may still be in flight
+          if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
           wait_lds();        // this wave's reads of stage CUR have all returned (the compiler cannot see the asm ones)
-          __syncthreads();   // ... everyone's part; and every wave is done reading stage CUR
+          // ... everyone's part; and every wave is done reading stage CUR.  The bare barrier instruction:
+          // __syncthreads() comes with a fence in front of which the compiler drains every fetch in
+          // flight (vmcnt(0)), which would expose the whole memory latency at each tile.  What has
+          // to be complete at this point is exactly what the two waits above ask for.
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
         }
         if (q == 0) wait_frags(fa[s & 1], fb[s & 1]);   // fragments of this step (read under the previous one) are complete
         // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
         // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
         MI::run(acc[q / TNI][q % TNI], fb[s & 1][q % TNI].get(), fa[s & 1][q / TNI].get());
-        if constexpr (HN) {
 #pragma unroll
-          for (int i = 0; i < NFETCH; ++i)
-            if (BAR + (i * TAIL) / NFETCH == slot) fetch_item(i, tbn, IntC<CUR>());
+        for (int i = 0; i < NFETCH; ++i) {
+          const int pos = BAR + (i * SPREAD) / NFETCH;          // position on the time line that starts at this tile
+          if (HN && pos == slot) fetch_item(i, tbn, IntC<CUR>());
+          if (HP && pos - MT == slot) fetch_item(i, tbp, IntC<PRV>());
         }
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
@@ -803,15 +823,22 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       for (int j = 0; j < TNI; ++j) fb[0][j] = fb[1][j];
     }
   };
-  // main part: groups of NST tiles, every tile with both successors; the rest is unrolled with the
-  // right flags at compile time (KT is a constant)
-  constexpr int NG = (KT >= 2 * NST) ? (KT - 2 * NST) / NST + 1 : 0;
+  // Tile 0 first (nothing of an earlier period to continue); then groups of NST tiles that have every
+  // neighbour; the rest is unrolled with the right flags at compile time (KT is a constant).
+  // tiles_ahead(T): how many tiles behind tile T+1 have been issued when tile T reaches its barrier
+  // (the prologue issued tiles 0..NST-1, tile t issues or completes the issue of tile t-1+NST)
+  tile(0, IntC<0>(), BoolC<(1 < KT)>(), BoolC<(NST < KT)>(), BoolC<false>(), IntC<tiles_ahead(0)>());
+  constexpr int NFULL = KT - NST - 1 > 0 ? KT - NST - 1 : 0;   // tiles 1 .. KT-NST-1 have kt+NST < KT
+  constexpr int NG = NFULL / NST;
   for (int g = 0; g < NG; ++g) {
-    static_for<0, NST>([&](auto sc) { tile(g * NST + decltype(sc)::value, sc, BoolC<true>(), BoolC<true>()); });
+    static_for<0, NST>([&](auto sc) {
+      constexpr int S = decltype(sc)::value;
+      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>());
+    });
   }
-  static_for<NG * NST, KT>([&](auto tc) {
+  static_for<1 + NG * NST, KT>([&](auto tc) {
     constexpr int T = decltype(tc)::value;
-    tile(T, IntC<T % NST>(), BoolC<(T + 1 < KT)>(), BoolC<(T + NST < KT)>());
+    tile(T, IntC<T % NST>(), BoolC<(T + 1 < KT)>(), BoolC<(T + NST < KT)>(), BoolC<(T - 1 + NST < KT)>(), IntC<tiles_ahead(T)>());
   });
 
   // ---- epilogue --------------------------------------------------------------------------------

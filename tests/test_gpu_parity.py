@@ -98,6 +98,18 @@ HALF_CASES = [
                          shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-out16", dict(M=256, N=256, K=128, dtype=2, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
                               shared_prefetch=1, reg_prefetch=1)),
+    # long K: the steady-state part of the direct-staging K loop (groups of NST tiles) with 4, 2, 3 and 4
+    # LDS stages, tile counts that leave 1..NST tiles for the unrolled rest
+    ("f16-direct-longk-4st", dict(M=256, N=256, K=2048, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8,
+                                  BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-longk-2st", dict(M=256, N=512, K=1024, dtype=2, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=16, TN=16,
+                                  BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-longk-3st-at1", dict(M=512, N=256, K=1088, dtype=2, dtype_c=4, is_atrans=1, BM=256, BN=128, TM=16,
+                                      TN=8, BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-direct-longk-bk32", dict(M=512, N=256, K=1056, dtype=3, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=16, TN=16,
+                                    BK=32, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-longk-8w", dict(M=256, N=256, K=1600, dtype=2, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=8, TN=16,
+                                 BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("bf16-at0", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=0, BK=32)),
     ("bf16-at1-lsu2", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=1, BK=64, lsu=2)),
 ]
@@ -106,8 +118,8 @@ HALF_CASES = [
 @pytest.mark.parametrize("tag,kw", HALF_CASES, ids=[c[0] for c in HALF_CASES])
 @pytest.mark.parametrize("kind", [MFMA, SIMT], ids=["mfma", "simt"])
 def test_exact_small_integers_16bit(oracle, tag, kw, kind):
-    """Integers in [-4,4] are exact in fp16/bf16; sums of <=256 products of them (|sum| <= 4096) are
-    exact in fp32 and representable in fp16 up to 2048 -> lim=2 keeps the fp16-output case exact."""
+    """Integers in [-2,2] are exact in fp16/bf16 and sums of K <= 2048 products of them (|sum| <= 8192)
+    are exact in fp32; the fp16-output cases keep K <= 256 so that their sums (<= 1024) stay exact."""
     cfg = make_config(**kw)
     M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
     lim = 2
