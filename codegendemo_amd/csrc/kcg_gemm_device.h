@@ -466,12 +466,26 @@ template <> struct Mfma<_Float16, 32> {
   __device__ __forceinline__ static void run(Acc& c, const Frag& a, const Frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  // the same instruction with the accumulator tied to its own registers (accumulation registers):
+  // left to itself the register allocator gives some of these instructions a fresh destination and
+  // copies accumulators around the loop.  The compiler does not see a matrix-core instruction here:
+  // the caller keeps dependent uses of c (as accumulator input or as plain data) far enough away.
+  __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
 };
 template <> struct Mfma<_Float16, 16> {
   typedef floatx4 Acc;
   typedef halfx8 Frag;
   __device__ __forceinline__ static void run(Acc& c, const Frag& a, const Frag& b) {
     c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  // the same instruction with the accumulator tied to its own registers (accumulation registers):
+  // left to itself the register allocator gives some of these instructions a fresh destination and
+  // copies accumulators around the loop.  The compiler does not see a matrix-core instruction here:
+  // the caller keeps dependent uses of c (as accumulator input or as plain data) far enough away.
+  __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
 };
 template <> struct Mfma<__bf16, 32> {
@@ -480,12 +494,26 @@ template <> struct Mfma<__bf16, 32> {
   __device__ __forceinline__ static void run(Acc& c, const Frag& a, const Frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // the same instruction with the accumulator tied to its own registers (accumulation registers):
+  // left to itself the register allocator gives some of these instructions a fresh destination and
+  // copies accumulators around the loop.  The compiler does not see a matrix-core instruction here:
+  // the caller keeps dependent uses of c (as accumulator input or as plain data) far enough away.
+  __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
 };
 template <> struct Mfma<__bf16, 16> {
   typedef floatx4 Acc;
   typedef bf16x8 Frag;
   __device__ __forceinline__ static void run(Acc& c, const Frag& a, const Frag& b) {
     c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  // the same instruction with the accumulator tied to its own registers (accumulation registers):
+  // left to itself the register allocator gives some of these instructions a fresh destination and
+  // copies accumulators around the loop.  The compiler does not see a matrix-core instruction here:
+  // the caller keeps dependent uses of c (as accumulator input or as plain data) far enough away.
+  __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
 };
 
@@ -518,12 +546,53 @@ struct LdsTile {
 // =============================================================================================
 typedef short short4v __attribute__((ext_vector_type(4)));
 
+// Static schedule of the fragment reads of one k-step of the direct-staging kernel (see its K loop):
+// which slot reads which B fragment of the next step, and how many LDS read instructions issued after
+// the fragments a row needs may still be in flight when that row starts.
+template <int TMI, int TNI, int DA, int NAI, int NBI>
+struct StreamPlan {
+  static constexpr int NM = TMI * TNI;
+  static constexpr int RB = TMI - DA;                              // first row whose side work belongs to the next step
+  static constexpr int BW0 = RB * TNI;                             // B reads: slots [BW0, BW1)
+  static constexpr int BW1 = DA > 1 ? (TMI - 1) * TNI : NM;
+  static constexpr int slot_b(int j) { return BW0 + (j * (BW1 - BW0)) / TNI; }
+  // issue times in half slots: a row's A read comes first in its slot, a B read follows the
+  // matrix-core instruction of its slot
+  static constexpr int time_a(int step, int row) { return (step * NM + (row - DA) * TNI) * 2; }
+  static constexpr int time_b(int step, int j) { return ((step - 1) * NM + slot_b(j)) * 2 + 1; }
+  static constexpr int allowed(int row) {
+    const int step = 2;
+    const int now = (step * NM + row * TNI) * 2 - 1;               // just before this row's own A read
+    int need = time_a(step, row);
+    if (row == 0)
+      for (int j = 0; j < TNI; ++j) need = cmax(need, time_b(step, j));
+    int n = 0;
+    for (int st = 0; st <= step + 1; ++st) {
+      for (int r = 0; r < TMI; ++r) {
+        const int t = time_a(st, r);
+        if (t > need && t < now) n += NAI;
+      }
+      for (int j = 0; j < TNI; ++j) {
+        const int t = time_b(st, j);
+        if (t > need && t < now) n += NBI;
+      }
+    }
+    return cmin(n, 15);                                            // the counter field has 4 bits; less is safe
+  }
+};
+
 template <class C>
 struct DirectPlan {
   typedef typename C::TA T;
   static constexpr int ES = (int)sizeof(T);
   static constexpr int WM = C::BM / C::BLM, WN = C::BN / C::BLN;
-  static constexpr int MF = (WM % 32 == 0 && WN % 32 == 0) ? 32 : 16;
+  // 16x16x32 instructions where the K tile allows: on fp16/bf16 data with realistic bit activity a
+  // gfx950 sustains about 16 % more flops with them than with 32x32x16 at its power limit
+#ifndef KCG_DIRECT_MF
+#define KCG_DIRECT_MF 0               /* 16 or 32 forces the matrix-core tile of the direct-staging kernel */
+#endif
+  static constexpr int MF = KCG_DIRECT_MF ? KCG_DIRECT_MF
+                            : (C::BK % 32 == 0 || WM % 32 != 0 || WN % 32 != 0) ? 16 : 32;
   static constexpr int KS = 8 * (64 / MF);
   static constexpr int NW = C::BLM * C::BLN;
   static constexpr int NM = (WM / MF) * (WN / MF);
@@ -531,13 +600,15 @@ struct DirectPlan {
   static constexpr bool pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
   static constexpr bool ELIGIBLE =
       ES == 2 && !C::EDGE && C::SHMP && C::REGP && C::LC != 0 && C::LSU == 1 && C::GLW_A == 8 && C::GLW_B == 8 &&
-      SPW > 0 && SPW * NM >= 4 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
+      SPW > 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
       (C::BM * C::BK / 8) % (64 * NW) == 0 && (C::BN * C::BK / 8) % (64 * NW) == 0 && (C::M % 8 == 0) &&
       (C::N % 8 == 0) && (C::K % 8 == 0) && 2 * (C::BM + C::BN) * C::BK * 2 <= 160 * 1024;
-  // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles)
+  // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles); an even number
+  // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
   static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * 2;
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
-  static constexpr int NST = NST_FIT < 2 ? 2 : (NST_FIT > 4 ? 4 : NST_FIT);
+  static constexpr int NST_CAP = NST_FIT < 2 ? 2 : (NST_FIT > 4 ? 4 : NST_FIT);
+  static constexpr int NST = (SPW % 2 == 1 && NST_CAP % 2 == 1) ? NST_CAP - 1 : NST_CAP;
   // the host picks the path (it must size dynamic LDS accordingly); both sides have to agree
   static_assert(ELIGIBLE == C::DIRECT, "host and device disagree on the direct-staging eligibility rule");
   static constexpr bool OK = C::DIRECT;
@@ -575,25 +646,17 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   block_coords<C>(blockIdx.x, by, bx);
   const int m0 = by * BM, n0 = bx * BN;
 
-  // The stages are separate LDS objects on purpose: the compiler then knows that a fragment read
-  // from one stage cannot alias an in-flight fetch into the other and does not wait for the fetch.
-  // (For the same reason the K loop below is unrolled by two, so every access names its stage.)
+  // One LDS array holds the NST stages.  (No LDS access of this kernel is visible to the compiler as a
+  // load: otherwise it would have to assume that the load may touch a stage a fetch is in flight to
+  // and drain all fetches in front of it.)
   constexpr int NST = P::NST;
-  __shared__ __attribute__((aligned(1024))) char lds_stage0[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char lds_stage1[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char lds_stage2[NST > 2 ? STAGE_BYTES : 16];
-  __shared__ __attribute__((aligned(1024))) char lds_stage3[NST > 3 ? STAGE_BYTES : 16];
+  __shared__ __attribute__((aligned(1024))) char lds_all[NST * STAGE_BYTES];
   (void)smem;
-  auto stage_ptr = [&](auto stage_c) -> char* {
-    constexpr int S = decltype(stage_c)::value;
-    if constexpr (S == 0) return lds_stage0;
-    else if constexpr (S == 1) return lds_stage1;
-    else if constexpr (S == 2) return lds_stage2;
-    else return lds_stage3;
-  };
+  auto stage_ptr = [&](auto stage_c) -> char* { return lds_all + decltype(stage_c)::value * STAGE_BYTES; };
 
-  // swizzle of a row-contiguous tile: rows k..k+3 of a transposing read must not share banks
-  auto swz_n = [](int k, int nch) { return ((k & 3) << 2) & (nch - 1); };
+  // swizzle of a row-contiguous tile (chunk index ^= swz_n(row)): the rows that one pass of a transposing
+  // read touches (k..k+3, and k+8..k+11 with 16-wide matrix-core tiles) must not share banks
+  auto swz_n = [](int k, int nch) { return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & (nch - 1); };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
@@ -652,19 +715,17 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int NFETCH = NIA + NIB;
 
   // ---- fragments -----------------------------------------------------------------------------
+  // Every fragment read is issued as inline assembly.  As builtins or plain loads the compiler could
+  // not tell that they do not touch the stage a fetch is in flight to and would drain all fetches
+  // (vmcnt(0)) in front of them; it would also insert its own LDS waits, which know nothing of the
+  // reads it cannot see.  The price: the compiler does not know that these reads are asynchronous, so
+  // (1) the K loop counts the reads in flight itself and waits with s_waitcnt lgkmcnt(n) in front of the
+  // matrix-core instructions that consume a fragment, and (2) a fragment stays in the very registers
+  // the read instruction wrote (never a copy made before the data has arrived) until it is consumed.
   const int frow = lane % MF, fgrp = lane / MF;
   const int tx = lane % 16;                          // lane inside its 16-lane transposing group
-  const int tsub = (lane / 16) % (MF / 16);          // which 16-column half of the MFMA tile
-  // row-contiguous tile: 8 k values of column (rowbase + lane%MF), k = kb .. kb+7, from two 4x16 blocks
-  // The transposing read is issued as inline assembly: as a builtin the compiler cannot tell that it
-  // does not touch the stage a fetch is in flight to, and would drain all fetches (vmcnt(0)) in front
-  // of every such read.  The price: the compiler does not know these reads are asynchronous either,
-  // so the loop below waits for them itself (wait_frags) before the matrix-core step that consumes them.
-  // A fragment read with the transposing instruction lives in two 64-bit halves until the matrix-core
-  // instruction that consumes it: those reads are asynchronous and invisible to the compiler, so
-  // their destination registers must stay the asm outputs themselves (never a copy made before the
-  // data has arrived).  Fragments read with an ordinary 128-bit load are one value.
-  struct FragTr {
+  const int tsub = (lane / 16) % (MF / 16);          // which 16-column half of the matrix-core tile
+  struct FragTr {                                    // two transposing 64-bit reads
     u32x2 h[2];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
     __device__ __forceinline__ Frag get() const {
@@ -672,47 +733,64 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       return __builtin_bit_cast(Frag, v);
     }
   };
-  struct FragLd {
+  struct FragLd {                                    // one 128-bit read
     u32x4 q;
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(q)); }
     __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
   };
   typedef typename Select<AK, FragLd, FragTr>::type FragA;
   typedef FragTr FragB;
-  auto read_tr = [&](const char* tile, int nch, int rowbase, int kb, FragTr* dst) {
+  // LDS address of a fragment read = a per-lane base that never changes (one register per fragment
+  // column block of a row-contiguous tile, one per k-step of a k-contiguous tile) + a compile-time
+  // offset (stage, k-step, fragment row block) that goes into the instruction's 16-bit offset field;
+  // what does not fit the field is added to the base in units of 64 KiB.
+  const unsigned lds0 = (unsigned)(unsigned long)lds_all;
+  // row-contiguous tile (nch chunks per row at byte offset toff of a stage): a lane reads 8 k values of
+  // column rowbase + lane%MF, k = kb .. kb+7 with kb = s*KS + 8*fgrp, from two 4(k) x 16(n) blocks.
+  // The swizzle of row k depends on the lane only (k&3 = (tx/4)&3, (k>>3)&1 = fgrp&1: KS is a multiple of 16).
+  auto tr_lane_base = [&](int toff, int nch, int rowbase) {
     const int n = rowbase + 16 * tsub + 4 * (tx % 4);
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int k = kb + 4 * t + tx / 4;
-      const unsigned addr = (unsigned)(unsigned long)(tile + ((k * nch + ((n / 8) ^ swz_n(k, nch))) * 16) + (n % 8) * 2);
-      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst->h[t]) : "v"(addr));
-    }
+    const int k = 8 * fgrp + tx / 4;
+    return lds0 + (unsigned)(toff + (k * nch + ((n / 8) ^ swz_n(k, nch))) * 16 + (n % 8) * 2);
   };
-  // lgkmcnt(0): every LDS read issued so far (compiler-visible or not) has returned.  The empty asm
-  // statements that follow make the fragments "outputs" of the wait, so the matrix-core instructions
-  // that consume them cannot be scheduled in front of it (volatile asm keeps its program order).
-  auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
-  auto wait_frags = [&](FragA* a, FragB* b) {
-    wait_lds();
+  unsigned b_lane[TNI];
 #pragma unroll
-    for (int i = 0; i < TMI; ++i) a[i].pin();
+  for (int j = 0; j < TNI; ++j) b_lane[j] = tr_lane_base(A_BYTES, NCHB, wx * WN + j * MF);
+  constexpr int NALANE = AK ? SPW : TMI;
+  unsigned a_lane[NALANE];
+  if constexpr (AK) {
 #pragma unroll
-    for (int j = 0; j < TNI; ++j) b[j].pin();
+    for (int st = 0; st < SPW; ++st)
+      a_lane[st] = lds0 + (unsigned)(LK::slot(wy * WM + frow, st * KH + fgrp) * 16);   // swizzle: row%16 = frow%16 only
+  } else {
+#pragma unroll
+    for (int i = 0; i < TMI; ++i) a_lane[i] = tr_lane_base(0, NCHA, wy * WM + i * MF);
+  }
+  auto split_base = [](unsigned lane_base, int imm) { return lane_base + (unsigned)(imm / 65536) * 65536u; };
+  auto read_tr = [&](unsigned lane_base, auto imm_c, auto nch_c, FragTr* dst) {
+    constexpr int IMM0 = decltype(imm_c)::value;
+    constexpr int IMM1 = IMM0 + 4 * decltype(nch_c)::value * 16;      // second block: four rows further
+    const unsigned base0 = split_base(lane_base, IMM0), base1 = split_base(lane_base, IMM1);
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[0]) : "v"(base0), "n"(IMM0 % 65536));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[1]) : "v"(base1), "n"(IMM1 % 65536));
   };
-  auto load_frag_item = [&](auto stage_c, int s, int f, FragA* fa, FragB* fb) {
-    const char* st = stage_ptr(stage_c);
-    if (f < TMI) {
-      if constexpr (AK) {
-        const int row = wy * WM + f * MF + frow;
-        fa[f].q = *(const u32x4*)(st + LK::slot(row, s * KH + fgrp) * 16);
-      } else {
-        read_tr(st, NCHA, wy * WM + f * MF, s * KS + 8 * fgrp, &fa[f]);
-      }
+  // fragment f of k-step s of the stage: s, f and the stage are compile-time constants (IntC)
+  auto load_a = [&](auto stage_c, auto s_c, auto f_c, FragA* dst) {
+    constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
+    if constexpr (AK) {
+      constexpr int IMM = ST * STAGE_BYTES + F * MF * CHK * 16;
+      const unsigned base = split_base(a_lane[S], IMM);
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst->q) : "v"(base), "n"(IMM % 65536));
     } else {
-      read_tr(st + A_BYTES, NCHB, wx * WN + (f - TMI) * MF, s * KS + 8 * fgrp, &fb[f - TMI]);
+      read_tr(a_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHA * 16>(), IntC<NCHA>(), dst);
     }
   };
-  constexpr int NF = TMI + TNI;
+  auto load_b = [&](auto stage_c, auto s_c, auto f_c, FragB* dst) {
+    constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
+    read_tr(b_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHB * 16>(), IntC<NCHB>(), dst);
+  };
+  // lgkmcnt(0): every LDS read issued so far has returned
+  auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
 
   Acc acc[TMI][TNI];
 #pragma unroll
@@ -721,24 +799,38 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     for (int j = 0; j < TNI; ++j)
 #pragma unroll
       for (int e = 0; e < (int)(sizeof(Acc) / sizeof(float)); ++e) acc[i][j][e] = 0.0f;
+  // The zeros must be in their registers here and now: left alone the compiler writes them right in
+  // front of the first matrix-core instruction of each accumulator, and that instruction (which the
+  // compiler does not recognise as one, see Mfma::run_tied) would need wait states after such a write.
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j) asm volatile("" : "+a"(acc[i][j]));
+  asm volatile("s_nop 7" ::: "memory");
 
-  // ---- K loop: NST LDS stages; the barrier stands in front of the last step of a tile -----------------
-  // Schedule constants (time line = the MT matrix-core groups of a tile).  The defaults can be
-  // overridden per build with -DKCG_SCHED_...=n through $KCG_EXTRA_FLAGS when exploring schedules.
-#ifndef KCG_SCHED_BAR_Q
-#define KCG_SCHED_BAR_Q 0             /* barrier stands in front of this group of the last step */
+  // ---- K loop ----------------------------------------------------------------------------------
+  // Time line of a k-step: its NM = TMI x TNI matrix-core instructions, row by row (row i: fragment
+  // A_i against B_0..B_TNI-1).  Side work is pinned to slots of that time line:
+  //   * the A fragment that row i+DA needs is read when row i starts (rows >= TMI: rows of the next
+  //     step); it replaces the fragment of a row that is done, so A takes TMI fragments of registers;
+  //   * the B fragments of the next step are read into the other half of a double buffer in the slots
+  //     slot_b(j) of rows RB..TMI-2 (RB = TMI-DA);
+  //   * in the last step of a tile the barrier stands where row RB starts: all reads of this stage
+  //     have been issued by then, and everything read from there on belongs to the next tile;
+  //   * fetches: see below.
+  // LDS reads return in order, so "fragment X has arrived" is "at most n reads issued after X are
+  // still in flight"; n is a compile-time property of this schedule (StreamPlan::allowed).
+#ifndef KCG_SCHED_A_AHEAD
+#define KCG_SCHED_A_AHEAD 0           /* rows an A fragment is read ahead of its use; 0 = TMI/2 */
 #endif
-#ifndef KCG_SCHED_FSPAN_PCT
-#define KCG_SCHED_FSPAN_PCT 50        /* next-step fragment reads are spread over this share of a step */
-#endif
-#ifndef KCG_SCHED_NSPAN_PCT
-#define KCG_SCHED_NSPAN_PCT 50        /* next-tile fragment reads: share of the groups behind the barrier */
-#endif
+  constexpr int DA = cmax(1, cmin(TMI - 1, KCG_SCHED_A_AHEAD > 0 ? KCG_SCHED_A_AHEAD : TMI / 2));
+  typedef StreamPlan<TMI, TNI, DA, (AK ? 1 : 2), 2> SP;
+  constexpr int RB = SP::RB;
   constexpr int MT = SPW * NM;
-  constexpr int BAR = (SPW - 1) * NM + cmin(NM - 1, cmax(0, KCG_SCHED_BAR_Q));
-  constexpr int FSPAN = cmax(1, (NM * KCG_SCHED_FSPAN_PCT) / 100);
-  constexpr int NSPAN = cmax(1, ((MT - BAR) * KCG_SCHED_NSPAN_PCT) / 100);
+  constexpr int BAR = (SPW - 1) * NM + RB * TNI;
   constexpr int TAIL = MT - BAR;
+  static_assert(TMI >= 2, "the streaming schedule needs two rows of matrix-core tiles per wave");
+  static_assert((NST * SPW) % 2 == 0, "B double buffer: the parity of a step must follow from its stage");
   // s_waitcnt vmcnt(n), everything else unconstrained: n fetches of this wave may still be in flight
   static_assert((NST - 2) * NFETCH < 64, "vmcnt has 6 bits");
   auto vmcnt_only = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
@@ -758,10 +850,11 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t);
     }
   });
-  FragA fa[2][TMI];
+  FragA fa[TMI];
   FragB fb[2][TNI];
-#pragma unroll
-  for (int f = 0; f < NF; ++f) load_frag_item(IntC<0>(), 0, f, fa[0], fb[0]);
+  static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
+  static_for<0, DA>([&](auto i) { load_a(IntC<0>(), IntC<0>(), i, &fa[decltype(i)::value]); });
+  wait_lds();   // the counted waits of the loop assume that nothing older than its own reads is in flight
 
   // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists; HP: the
   // fetch of tile kt-1+NST, begun behind the previous tile's barrier, is still being issued.
@@ -779,16 +872,22 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     constexpr bool HP = decltype(hasp)::value && SPREAD > TAIL;
     const TileBase tbn = tile_base(HN ? kt + NST : 0);
     const TileBase tbp = tile_base(HP ? kt - 1 + NST : 0);
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-#pragma unroll
-      for (int q = 0; q < NM; ++q) {
-        const int slot = s * NM + q;
-        if (slot == BAR) {
+    static_for<0, SPW>([&](auto s_c) {
+      constexpr int S = decltype(s_c)::value;
+      constexpr bool LAST = (S == SPW - 1);
+      constexpr int PB = (CUR * SPW + S) & 1;       // half of the B double buffer this step computes from
+      constexpr bool NEXT = !LAST || H1;            // a next step exists, its fragments are read under this one
+      static_for<0, TMI>([&](auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        // the fragments of this row have arrived.  Without a next step the reads the count relies on
+        // are not issued: wait for everything instead.
+        if constexpr (NEXT) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(SP::allowed(I)) : "memory");
+        else wait_lds();
+        if constexpr (LAST && I == RB) {
           // tile kt+1 has landed (this wave's part): of the fetches issued so far only those of the
           // tiles behind it may still be in flight
           if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
-          wait_lds();        // this wave's reads of stage CUR have all returned (the compiler cannot see the asm ones)
+          wait_lds();        // this wave's reads of stage CUR have all returned
           // ... everyone's part; and every wave is done reading stage CUR.  The bare barrier instruction:
           // __syncthreads() comes with a fence in front of which the compiler drains every fetch in
           // flight (vmcnt(0)), which would expose the whole memory latency at each tile.  What has
@@ -797,31 +896,39 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
         }
-        if (q == 0) wait_frags(fa[s & 1], fb[s & 1]);   // fragments of this step (read under the previous one) are complete
-        // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
-        // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
-        MI::run(acc[q / TNI][q % TNI], fb[s & 1][q % TNI].get(), fa[s & 1][q / TNI].get());
+        // the empty asm statements make the fragments "outputs" of the wait: the matrix-core
+        // instructions that consume them cannot be scheduled in front of it
+        fa[I].pin();
+        if constexpr (I == 0) {
 #pragma unroll
-        for (int i = 0; i < NFETCH; ++i) {
-          const int pos = BAR + (i * SPREAD) / NFETCH;          // position on the time line that starts at this tile
-          if (HN && pos == slot) fetch_item(i, tbn, IntC<CUR>());
-          if (HP && pos - MT == slot) fetch_item(i, tbp, IntC<PRV>());
+          for (int j = 0; j < TNI; ++j) fb[PB][j].pin();
         }
+        if constexpr (I + DA < TMI) load_a(IntC<CUR>(), IntC<S>(), IntC<I + DA>(), &fa[I + DA]);
+        else if constexpr (!LAST) load_a(IntC<CUR>(), IntC<S + 1>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
+        else if constexpr (H1) load_a(IntC<NXT>(), IntC<0>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
+        static_for<0, TNI>([&](auto j_c) {
+          constexpr int J = decltype(j_c)::value;
+          constexpr int slot = S * NM + I * TNI + J;
+          // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
+          // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
+          MI::run_tied(acc[I][J], fb[PB][J].get(), fa[I].get());
+          static_for<0, TNI>([&](auto jj_c) {
+            constexpr int JJ = decltype(jj_c)::value;
+            if constexpr (SP::slot_b(JJ) == I * TNI + J) {
+              if constexpr (!LAST) load_b(IntC<CUR>(), IntC<S + 1>(), jj_c, &fb[PB ^ 1][JJ]);
+              else if constexpr (H1) load_b(IntC<NXT>(), IntC<0>(), jj_c, &fb[PB ^ 1][JJ]);
+            }
+          });
 #pragma unroll
-        for (int f = 0; f < NF; ++f) {
-          if (s + 1 < SPW && (f * FSPAN) / NF == q)
-            load_frag_item(IntC<CUR>(), s + 1, f, fa[(s + 1) & 1], fb[(s + 1) & 1]);
-          if (H1 && BAR + (f * NSPAN) / NF == slot) load_frag_item(IntC<NXT>(), 0, f, fa[SPW & 1], fb[SPW & 1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    if constexpr (SPW % 2 == 1) {
-#pragma unroll
-      for (int i = 0; i < TMI; ++i) fa[0][i] = fa[1][i];
-#pragma unroll
-      for (int j = 0; j < TNI; ++j) fb[0][j] = fb[1][j];
-    }
+          for (int f = 0; f < NFETCH; ++f) {
+            const int pos = BAR + (f * SPREAD) / NFETCH;          // position on the time line that starts at this tile
+            if (HN && pos == slot) fetch_item(f, tbn, IntC<CUR>());
+            if (HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>());
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      });
+    });
   };
   // Tile 0 first (nothing of an earlier period to continue); then groups of NST tiles that have every
   // neighbour; the rest is unrolled with the right flags at compile time (KT is a constant).
@@ -841,6 +948,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     tile(T, IntC<T % NST>(), BoolC<(T + 1 < KT)>(), BoolC<(T + NST < KT)>(), BoolC<(T - 1 + NST < KT)>(), IntC<tiles_ahead(T)>());
   });
 
+  // the last matrix-core results must have left the pipeline before the epilogue reads them (the
+  // compiler, which normally inserts these wait states, does not know the instructions above)
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   // ---- epilogue --------------------------------------------------------------------------------
   // With swapped operands a 32x32 accumulator holds, per lane, row m = lane%32 and columns
   // n = 8*g + 4*(lane/32) + {0..3} for g = 0..3 (16x16: row lane%16, columns 4*(lane/16) + {0..3}).
