@@ -383,6 +383,24 @@ int kcg_instantiation_source(const kcg_matmul_cfg* cfg, int kind, char* out, int
   return copy_out(kcg::instantiation_source(c, k, env_flag("KCG_XCD_REMAP", true)), out, out_len);
 }
 
+// Scratch (private segment) bytes per lane of the kernel in a code object, from its metadata note:
+// the msgpack key ".private_segment_fixed_size" is followed by its unsigned value.  -1 when the key is
+// not there (the caller then does not know).
+static long code_object_scratch_bytes(const std::vector<char>& code) {
+  static const char key[] = ".private_segment_fixed_size";
+  const size_t klen = sizeof(key) - 1;
+  for (size_t i = 0; i + klen + 1 <= code.size(); ++i) {
+    if (memcmp(code.data() + i, key, klen) != 0) continue;
+    const unsigned char* p = reinterpret_cast<const unsigned char*>(code.data()) + i + klen;
+    const size_t left = code.size() - (i + klen);
+    if (left >= 1 && p[0] <= 0x7f) return p[0];
+    if (left >= 2 && p[0] == 0xcc) return p[1];
+    if (left >= 3 && p[0] == 0xcd) return (p[1] << 8) | p[2];
+    if (left >= 5 && p[0] == 0xce) return ((long)p[1] << 24) | (p[2] << 16) | (p[3] << 8) | p[4];
+  }
+  return -1;
+}
+
 int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, kcg_kernel_info* out) {
   if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
   kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
@@ -458,6 +476,15 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   if (r == HIPRTC_SUCCESS) r = RTCF(hiprtcGetCode)(prog, code.data());
   RTCF(hiprtcDestroyProgram)(&prog);
   if (r != HIPRTC_SUCCESS || n == 0) return fail(KCG_ERR_COMPILE, "hiprtc returned no code object");
+  // The direct-staging kernel reads LDS with instructions the compiler does not know to be
+  // asynchronous: a fragment register spilled to scratch memory would be stored before its data has
+  // arrived.  Such a build is refused (and not cached) instead of returning wrong products.
+  if (k == KCG_KIND_MFMA && kcg::mfma_direct(c)) {
+    const long scratch = code_object_scratch_bytes(code);
+    if (scratch > 0)
+      return fail(KCG_ERR_COMPILE, "direct-staging kernel " + name + " needs " + std::to_string(scratch) +
+                                       " bytes of scratch memory per lane (register spills); use a smaller tile");
+  }
   if (!write_file_atomic(path, code.data(), code.size())) return fail(KCG_ERR_IO, "cannot write " + path);
   if (env_flag("KCG_KEEP_SOURCE", false)) {
     std::string sp = dir + "/" + name + "." + hex + ".hip";

@@ -821,9 +821,11 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // LDS reads return in order, so "fragment X has arrived" is "at most n reads issued after X are
   // still in flight"; n is a compile-time property of this schedule (StreamPlan::allowed).
 #ifndef KCG_SCHED_A_AHEAD
-#define KCG_SCHED_A_AHEAD 0           /* rows an A fragment is read ahead of its use; 0 = TMI/2 */
+#define KCG_SCHED_A_AHEAD 0           /* rows an A fragment is read ahead of its use; 0 = TMI-1 */
 #endif
-  constexpr int DA = cmax(1, cmin(TMI - 1, KCG_SCHED_A_AHEAD > 0 ? KCG_SCHED_A_AHEAD : TMI / 2));
+  // (the further ahead, the earlier the barrier stands in the last step and the more room the fetches
+  // behind it have; measured best at the maximum)
+  constexpr int DA = cmax(1, cmin(TMI - 1, KCG_SCHED_A_AHEAD > 0 ? KCG_SCHED_A_AHEAD : TMI - 1));
   typedef StreamPlan<TMI, TNI, DA, (AK ? 1 : 2), 2> SP;
   constexpr int RB = SP::RB;
   constexpr int MT = SPW * NM;
@@ -835,7 +837,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   static_assert((NST - 2) * NFETCH < 64, "vmcnt has 6 bits");
   auto vmcnt_only = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
   auto tiles_ahead = [](int t) {
-    const int last = cmin(KT - 1, cmax(t, 1) - 1 + NST);
+    const int last = cmin(KT - 1, t == 0 ? NST - 1 : t - 1 + NST);   // newest tile whose fetch has been issued
     return cmax(0, last - (t + 1));
   };
 
@@ -911,7 +913,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           constexpr int slot = S * NM + I * TNI + J;
           // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
           // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
-          MI::run_tied(acc[I][J], fb[PB][J].get(), fa[I].get());
+          // odd rows run right to left: neighbours on the time line always share one operand
+          constexpr int JC = (I & 1) ? TNI - 1 - J : J;
+          MI::run_tied(acc[I][JC], fb[PB][JC].get(), fa[I].get());
           static_for<0, TNI>([&](auto jj_c) {
             constexpr int JJ = decltype(jj_c)::value;
             if constexpr (SP::slot_b(JJ) == I * TNI + J) {

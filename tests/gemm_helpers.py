@@ -38,6 +38,11 @@ def run_gemm(config, a_mk, b_kn, kind=_native.KIND_AUTO, poison=True):
     b_dev = to_device(b_kn, ta)
     c_dev = torch.empty((kpm.M, kpm.N), dtype=tc, device="cuda:0")
     if poison:
+        # The same kernel first runs on NaN operands: LDS keeps its contents from launch to launch, so a
+        # kernel that reads a staging buffer before its data has landed would otherwise find the right
+        # values there whenever it (or a test with the same inputs) ran before, and pass by accident.
+        kernel.run(torch.full_like(a_dev, float("nan")), torch.full_like(b_dev, float("nan")), c_dev)
+        torch.cuda.synchronize()
         c_dev.fill_(float("nan"))
     kernel.run(a_dev, b_dev, c_dev)
     torch.cuda.synchronize()

@@ -86,7 +86,7 @@ HALF_CASES = [
                             shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-bk32", dict(M=256, N=384, K=224, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=32,
                              shared_prefetch=1, reg_prefetch=1)),
-    ("f16-direct-16x16", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=0, warp_layout=(4, 16), BM=64, BN=64,
+    ("f16-wl4x16-shmp", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=0, warp_layout=(4, 16), BM=64, BN=64,
                               BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-16x16-at1", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=1, warp_layout=(16, 4), BM=64,
                                   BN=64, BK=64, shared_prefetch=1, reg_prefetch=1)),
@@ -110,6 +110,16 @@ HALF_CASES = [
                                     BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-longk-8w", dict(M=256, N=256, K=1600, dtype=2, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=8, TN=16,
                                  BK=32, shared_prefetch=1, reg_prefetch=1)),
+    # the direct-staging kernel's other shapes: 32x32x16 instructions (K tile of 16), two rows of
+    # matrix-core tiles per wave (the minimum of its row-streaming loop), both A layouts
+    ("f16-direct-bk16-mf32", dict(M=256, N=256, K=400, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8,
+                                  BK=16, shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-direct-bk16-mf32-at1", dict(M=256, N=256, K=400, dtype=3, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8,
+                                       BK=16, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-2rows", dict(M=192, N=128, K=736, dtype=2, dtype_c=4, is_atrans=0, BM=64, BN=64, TM=4, TN=4,
+                              BK=32, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-2rows-at1", dict(M=192, N=128, K=736, dtype=2, dtype_c=4, is_atrans=1, BM=64, BN=64, TM=4, TN=4,
+                                  BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("bf16-at0", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=0, BK=32)),
     ("bf16-at1-lsu2", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=1, BK=64, lsu=2)),
 ]
