@@ -33,8 +33,8 @@ HBM_PEAK_GBS = 8000.0
 # by what the same counter read for a 256 MiB copy (FETCH x2.000, WRITE x1.000).  Keyed by the tile part
 # of the kernel name; a kernel that was not profiled reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x16_BTmnk256x256x32_BLmn2x2": (2 * 196747 + 65536) * 1024,
-    "DTabcfloat16xfloat16xfloat32_AT0_TTmn16x16_BTmnk256x256x64_BLmn2x2": (2 * 98706 + 66048) * 1024,
+    "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x16_BTmnk256x256x32_BLmn2x2": (2 * 196749 + 65536) * 1024,
+    "DTabcfloat16xfloat16xfloat32_AT0_TTmn16x16_BTmnk256x256x64_BLmn2x2": (2 * 98428 + 65536) * 1024,
 }
 
 
@@ -216,6 +216,16 @@ def main():
                        "roofline": {"bound": "mfma", "achieved": ach16, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
                                     "frac": ach16 / PEAK_TFLOPS["f16"], "traffic": measured_traffic(info16["kernel_name"]),
                                     "launch_ms": ms_launch16}}
+
+        # What the matrix pipeline alone sustains on this box (register operands, no memory traffic), on
+        # zeros and on data like the workload's: the stand-alone runner measures it in a child process.
+        # fp16 GEMMs on this part run at its power limit, so the second figure bounds any fp16 kernel.
+        runner = os.path.join(ROOT, "codegendemo_amd", "kcg_runner")
+        if os.path.exists(runner):
+            import subprocess
+            p = subprocess.run([runner, "--mfma-peak", "f16"], capture_output=True, text=True, timeout=120)
+            if p.returncode == 0:
+                out["fp16"]["mfma_only_sustained"] = json.loads(p.stdout.strip().splitlines()[-1])["mfma_peak"]
 
     if not args.no_cpu:
         base, panel, rows = cpu_baseline(a, b)

@@ -12,6 +12,12 @@
 //   kcg_runner M N K gridX blockX <code-object> <kernel-name> [ldsBytes] [dtypeCode] [isATrans]
 //       the reference runner's argument list (runkernel.cpp:63-66): launches an existing code object
 //
+//   kcg_runner --mfma-peak [dtype: f16|bf16]
+//       what the matrix pipeline of this GPU sustains with nothing else going on: a loop of independent
+//       matrix-core instructions on register operands, timed over ~0.3 s per case, for both 16-bit
+//       instruction shapes and for operands of all zeros and of normal(0, 0.5) values.  On a
+//       power-limited part the second figure is the ceiling of any GEMM on such data.
+//
 // Build: make -C codegendemo_amd/csrc runner      (hipcc --offload-arch=gfx950)
 #include <hip/hip_runtime.h>
 
@@ -64,6 +70,120 @@ __global__ void verify(const TC* __restrict__ C, const float* __restrict__ D, si
     atomicMin(first_bad, (unsigned long long)i);
   }
   if (err == err) atomicMax(max_err_bits, __float_as_uint(err));
+}
+
+// ---- sustained matrix-core rate: 64 independent accumulator tiles worth of work per iteration ----------
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 b8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef float f16_t __attribute__((ext_vector_type(16)));
+template <class V> struct PeakOp;
+template <> struct PeakOp<h8_t> {
+  __device__ static f4_t small(h8_t a, h8_t b, f4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+  __device__ static f16_t big(h8_t a, h8_t b, f16_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct PeakOp<b8_t> {
+  __device__ static f4_t small(b8_t a, b8_t b, f4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+  __device__ static f16_t big(b8_t a, b8_t b, f16_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+// opnd: 32 fragments of 8 values per lane (65536 lanes).  SMALL: 8x8 tiles of 16x16x32 over two k-steps;
+// otherwise 4x4 tiles of 32x32x16 over four k-steps: 2^22 flop per lane-iteration either way.
+template <class V, bool SMALL>
+__global__ __launch_bounds__(256) void mfma_peak(const V* __restrict__ opnd, float* sink, int iters) {
+  const int tid = blockIdx.x * 256 + threadIdx.x;
+  V frag[32];
+#pragma unroll
+  for (int f = 0; f < 32; ++f) frag[f] = opnd[(size_t)f * 65536 + tid];
+  float s = 0.f;
+  if constexpr (SMALL) {
+    f4_t acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] = f4_t{0, 0, 0, 0};
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+#pragma unroll
+        for (int q = 0; q < 64; ++q) {
+          acc[q / 8][q % 8] = PeakOp<V>::small(frag[k * 16 + 8 + q % 8], frag[k * 16 + q / 8], acc[q / 8][q % 8]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += acc[i][j][0] + acc[i][j][3];
+  } else {
+    f16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+          acc[q / 4][q % 4] = PeakOp<V>::big(frag[k * 8 + 4 + q % 4], frag[k * 8 + q / 4], acc[q / 4][q % 4]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s += acc[i][j][0] + acc[i][j][15];
+  }
+  if (s == 1234.5f) sink[tid] = s;   // keeps the loop alive; practically never true
+}
+
+template <class V, bool SMALL>
+static double run_mfma_peak(const V* d_opnd, float* d_sink) {
+  const int iters = 3000, launches = 50;           // 64 (or 4x16) instructions of 2^22/64 flop per lane-iteration
+  for (int i = 0; i < launches; ++i) hipLaunchKernelGGL((mfma_peak<V, SMALL>), dim3(256), dim3(256), 0, 0, d_opnd, d_sink, iters);
+  hipEvent_t e0, e1;
+  HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+  HIP_OK(hipEventRecord(e0, 0));
+  for (int i = 0; i < launches; ++i) hipLaunchKernelGGL((mfma_peak<V, SMALL>), dim3(256), dim3(256), 0, 0, d_opnd, d_sink, iters);
+  HIP_OK(hipEventRecord(e1, 0));
+  HIP_OK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  const double flops = (double)launches * iters * 128.0 * 16 * 16 * 32 * 2 * 4 * 256;   // per block: 4 waves
+  return flops / (ms * 1e-3) / 1e12;
+}
+
+template <class V, class E>
+static int mfma_peak_main(const char* tname) {
+  const size_t n = (size_t)32 * 65536;
+  std::vector<V> h(n);
+  V* d;
+  float* sink;
+  HIP_OK(hipMalloc(&d, n * sizeof(V)));
+  HIP_OK(hipMalloc(&sink, 65536 * sizeof(float)));
+  uint64_t st = 0x4B4347;
+  printf("{\"mfma_peak\": {\"dtype\": \"%s\"", tname);
+  for (int pass = 0; pass < 2; ++pass) {
+    for (size_t i = 0; i < n; ++i)
+      for (int e = 0; e < 8; ++e) {
+        float g = 0.f;
+        if (pass == 1) {   // normal(0, 0.5): Box-Muller on two uniforms
+          st = st * 6364136223846793005ull + 1442695040888963407ull;
+          const float u1 = ((float)(st >> 40) + 1.0f) / 16777217.0f;
+          st = st * 6364136223846793005ull + 1442695040888963407ull;
+          const float u2 = (float)(st >> 40) / 16777216.0f;
+          g = sqrtf(-2.0f * logf(u1)) * cosf(6.2831853f * u2) * 0.5f;
+        }
+        h[i][e] = (E)g;
+      }
+    HIP_OK(hipMemcpy(d, h.data(), n * sizeof(V), hipMemcpyHostToDevice));
+    const double small = run_mfma_peak<V, true>(d, sink), big = run_mfma_peak<V, false>(d, sink);
+    printf(", \"%s\": {\"16x16x32\": %.1f, \"32x32x16\": %.1f}", pass == 0 ? "zeros" : "normal(0,0.5)", small, big);
+  }
+  printf(", \"unit\": \"TFLOP/s\"}}\n");
+  HIP_OK(hipFree(d));
+  HIP_OK(hipFree(sink));
+  return 0;
 }
 
 static float lcg_uniform(uint64_t& s) {   // [-1, 1)
@@ -122,6 +242,10 @@ int main(int argc, char** argv) {
   float tol = 0.01f;   // the reference runner's tolerance (runkernel.cpp:34)
   int M = 0, N = 0, K = 0, dt = KCG_DT_FLOAT32, dtc = KCG_DT_FLOAT32, atrans = 1;
 
+  if (argc >= 2 && !strcmp(argv[1], "--mfma-peak")) {
+    if (argc >= 3 && !strcmp(argv[2], "bf16")) return mfma_peak_main<b8_t, __bf16>("bf16");
+    return mfma_peak_main<h8_t, _Float16>("f16");
+  }
   if (argc >= 3 && !strcmp(argv[1], "--config")) {
     std::string path = argv[2];
     for (int i = 3; i + 1 < argc; i += 2) {
@@ -157,8 +281,8 @@ int main(int argc, char** argv) {
     if (argc > 10) atrans = atoi(argv[10]);
     iters = 7;                                           // runkernel.cpp:104-108
   } else {
-    fprintf(stderr, "usage: %s --config file.json [--index i] [--kind auto|simt|mfma] [--iters n] [--tol t] [--compile-only 1]\n"
-                    "       %s M N K gridX blockX code-object kernel-name [ldsBytes] [dtypeCode] [isATrans]\n", argv[0], argv[0]);
+    fprintf(stderr, "usage: %s --mfma-peak [f16|bf16]\n       %s --config file.json [--index i] [--kind auto|simt|mfma] [--iters n] [--tol t] [--compile-only 1]\n"
+                    "       %s M N K gridX blockX code-object kernel-name [ldsBytes] [dtypeCode] [isATrans]\n", argv[0], argv[0], argv[0]);
     return 2;
   }
   if (dt == KCG_DT_FLOAT64 || (dtc != KCG_DT_FLOAT32)) {

@@ -58,3 +58,13 @@ def test_runner_reports_a_wrong_kernel():
     p = _run([1024, 1024, 1024, info["grid"][0], info["block"][0], info["code_path"], info["kernel_name"],
               info["lds_bytes"], 4, 1])
     assert p.returncode == 1 and "error!" in p.stdout and "no error!" not in p.stdout
+
+
+def test_runner_mfma_peak_mode():
+    """Sustained matrix-core rate on register operands: the figure on zeros is close to the published
+    peak, the one on normal(0, 0.5) data is lower on a power-limited part, never higher."""
+    p = _run(["--mfma-peak", "f16"])
+    assert p.returncode == 0
+    r = json.loads(p.stdout.strip().splitlines()[-1])["mfma_peak"]
+    for shape in ("16x16x32", "32x32x16"):
+        assert 500.0 < r["normal(0,0.5)"][shape] <= r["zeros"][shape] * 1.02 < 2516.6 * 1.05
