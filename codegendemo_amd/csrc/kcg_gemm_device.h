@@ -451,6 +451,12 @@ template <> struct Mfma<float, 32> {
 #pragma unroll
     for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], c, 0, 0, 0);
   }
+  // accumulator tied in place, see the 16-bit variants below.  Four dependent instructions in a row on
+  // one accumulator need no wait states between them (the compiler emits none for the builtin form either).
+  __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) asm volatile("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(c) : "v"(a[t]), "v"(b[t]));
+  }
 };
 template <> struct Mfma<float, 16> {
   typedef floatx4 Acc;
@@ -458,6 +464,12 @@ template <> struct Mfma<float, 16> {
   __device__ __forceinline__ static void run(Acc& c, const Frag& a, const Frag& b) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t], b[t], c, 0, 0, 0);
+  }
+  // accumulator tied in place, see the 16-bit variants below.  Four dependent instructions in a row on
+  // one accumulator need no wait states between them (the compiler emits none for the builtin form either).
+  __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+a"(c) : "v"(a[t]), "v"(b[t]));
   }
 };
 template <> struct Mfma<_Float16, 32> {
@@ -591,21 +603,25 @@ struct DirectPlan {
 #ifndef KCG_DIRECT_MF
 #define KCG_DIRECT_MF 0               /* 16 or 32 forces the matrix-core tile of the direct-staging kernel */
 #endif
+  static constexpr int G = 16 / ES;                               // elements per 16-byte chunk
+  static constexpr bool FITS32 = WM % 32 == 0 && WN % 32 == 0;
   static constexpr int MF = KCG_DIRECT_MF ? KCG_DIRECT_MF
-                            : (C::BK % 32 == 0 || WM % 32 != 0 || WN % 32 != 0) ? 16 : 32;
-  static constexpr int KS = 8 * (64 / MF);
+                            : ES == 2 ? ((C::BK % 32 == 0 || !FITS32) ? 16 : 32)
+                                      : (FITS32 ? 32 : 16);       // fp32: no such difference, the larger tile reads less
+  static constexpr int KS = G * (64 / MF);                        // k per step: one chunk per lane
   static constexpr int NW = C::BLM * C::BLN;
   static constexpr int NM = (WM / MF) * (WN / MF);
   static constexpr int SPW = (C::BK % KS == 0) ? C::BK / KS : 0;
   static constexpr bool pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
   static constexpr bool ELIGIBLE =
-      ES == 2 && !C::EDGE && C::SHMP && C::REGP && C::LC != 0 && C::LSU == 1 && C::GLW_A == 8 && C::GLW_B == 8 &&
+      (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && !C::EDGE && C::SHMP && C::REGP && C::LC != 0 &&
+      C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
       SPW > 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
-      (C::BM * C::BK / 8) % (64 * NW) == 0 && (C::BN * C::BK / 8) % (64 * NW) == 0 && (C::M % 8 == 0) &&
-      (C::N % 8 == 0) && (C::K % 8 == 0) && 2 * (C::BM + C::BN) * C::BK * 2 <= 160 * 1024;
+      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
+      (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024;
   // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles); an even number
   // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
-  static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * 2;
+  static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * ES;
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
   static constexpr int NST_CAP = NST_FIT < 2 ? 2 : (NST_FIT > 4 ? 4 : NST_FIT);
   static constexpr int NST = (SPW % 2 == 1 && NST_CAP % 2 == 1) ? NST_CAP - 1 : NST_CAP;
@@ -627,11 +643,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int TMI = WM / MF, TNI = WN / MF, NM = P::NM, NW = P::NW;
   constexpr int KT = K / BK;
   constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
-  constexpr int CHK = BK / 8;                           // chunks per row of a k-contiguous tile
-  constexpr int NCHA = BM / 8, NCHB = BN / 8;           // chunks per row of a row-contiguous tile
-  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int NIA = (BM * BK / 8) / (64 * NW);        // fetch instructions per wave and tile, operand A
-  constexpr int NIB = (BN * BK / 8) / (64 * NW);
+  constexpr int ES = P::ES, G = P::G;                   // element size; elements per 16-byte chunk
+  constexpr int CHK = BK / G;                           // chunks per row of a k-contiguous tile
+  constexpr int NCHA = BM / G, NCHB = BN / G;           // chunks per row of a row-contiguous tile
+  constexpr int A_BYTES = BM * BK * ES, B_BYTES = BN * BK * ES, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int NIA = (BM * BK / G) / (64 * NW);        // fetch instructions per wave and tile, operand A
+  constexpr int NIB = (BN * BK / G) / (64 * NW);
   typedef Mfma<T, MF> MI;
   typedef typename MI::Acc Acc;
   typedef typename MI::Frag Frag;
@@ -654,14 +671,20 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   (void)smem;
   auto stage_ptr = [&](auto stage_c) -> char* { return lds_all + decltype(stage_c)::value * STAGE_BYTES; };
 
-  // swizzle of a row-contiguous tile (chunk index ^= swz_n(row)): the rows that one pass of a transposing
-  // read touches (k..k+3, and k+8..k+11 with 16-wide matrix-core tiles) must not share banks
-  auto swz_n = [](int k, int nch) { return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & (nch - 1); };
+  // swizzle of a row-contiguous tile (chunk index ^= swz_n(row)).  16-bit: the rows that one pass of a
+  // transposing read touches (k..k+3, and k+8..k+11 with 16-wide matrix-core tiles) must not share banks.
+  // 32-bit: a fragment read is four 32-bit reads; in each, MF lanes read consecutive columns of one row
+  // and the 64/MF lane groups read rows 4 apart, which must fall into different bank ranges.
+  auto swz_n = [](int k, int nch) {
+    if constexpr (ES == 2) return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & (nch - 1);
+    else if constexpr (MF == 32) return (((k >> 2) & 1) << 3) & (nch - 1);
+    else return (((k >> 2) & 3) << 2) & (nch - 1);
+  };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
   // never changes: the K loop spends no vector instruction on addresses.
-  static_assert((long)BM * K * 2 < (1L << 31) && (long)BK * M * 2 < (1L << 31) && (long)BK * N * 2 < (1L << 31),
+  static_assert((long)BM * K * ES < (1L << 31) && (long)BK * M * ES < (1L << 31) && (long)BK * N * ES < (1L << 31),
                 "32-bit lane offsets");
   unsigned voff_a[NIA], voff_b[NIB];
 #pragma unroll
@@ -670,11 +693,11 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     if constexpr (AK) {
       const int row = s / CHK, cp = s % CHK;
       const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
-      voff_a[idx] = (unsigned)((row * K + c * 8) * 2);
+      voff_a[idx] = (unsigned)((row * K + c * G) * ES);
     } else {
       const int k = s / NCHA, cp = s % NCHA;
       const int c = cp ^ swz_n(k, NCHA);
-      voff_a[idx] = (unsigned)((k * M + c * 8) * 2);
+      voff_a[idx] = (unsigned)((k * M + c * G) * ES);
     }
   }
 #pragma unroll
@@ -682,12 +705,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     const int s = 64 * (wave * NIB + j) + lane;
     const int k = s / NCHB, cp = s % NCHB;
     const int c = cp ^ swz_n(k, NCHB);
-    voff_b[j] = (unsigned)((k * N + c * 8) * 2);
+    voff_b[j] = (unsigned)((k * N + c * G) * ES);
   }
   const char* const a_base = (const char*)(AK ? A + (long)m0 * K : A + m0);
   const char* const b_base = (const char*)(B + n0);
-  constexpr long A_KT_BYTES = AK ? (long)BK * 2 : (long)BK * M * 2;   // one K tile further
-  constexpr long B_KT_BYTES = (long)BK * N * 2;
+  constexpr long A_KT_BYTES = AK ? (long)BK * ES : (long)BK * M * ES;   // one K tile further
+  constexpr long B_KT_BYTES = (long)BK * N * ES;
   // The tile bases pass through an empty asm: the compiler must not fold the per-tile scalar part
   // into the per-lane part (it would hoist "base + lane offset" as a 64-bit vector value and add the
   // tile offset with vector instructions); kept apart, the fetch uses its scalar-base addressing form.
@@ -725,7 +748,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   const int frow = lane % MF, fgrp = lane / MF;
   const int tx = lane % 16;                          // lane inside its 16-lane transposing group
   const int tsub = (lane / 16) % (MF / 16);          // which 16-column half of the matrix-core tile
-  struct FragTr {                                    // two transposing 64-bit reads
+  struct FragTr {                                    // 16-bit, row-contiguous tile: two transposing 64-bit reads
     u32x2 h[2];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
     __device__ __forceinline__ Frag get() const {
@@ -733,29 +756,49 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       return __builtin_bit_cast(Frag, v);
     }
   };
-  struct FragLd {                                    // one 128-bit read
+  struct FragS4 {                                    // 32-bit, row-contiguous tile: four 32-bit reads
+    unsigned w[4];
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3])); }
+    __device__ __forceinline__ Frag get() const {
+      const u32x4 v = {w[0], w[1], w[2], w[3]};
+      return __builtin_bit_cast(Frag, v);
+    }
+  };
+  struct FragLd {                                    // k-contiguous tile: one 128-bit read
     u32x4 q;
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(q)); }
     __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
   };
-  typedef typename Select<AK, FragLd, FragTr>::type FragA;
-  typedef FragTr FragB;
+  typedef typename Select<ES == 2, FragTr, FragS4>::type FragRc;
+  typedef typename Select<AK, FragLd, FragRc>::type FragA;
+  typedef FragRc FragB;
+  constexpr int RC_READS = ES == 2 ? 2 : 4;          // LDS instructions per fragment of a row-contiguous tile
   // LDS address of a fragment read = a per-lane base that never changes (one register per fragment
   // column block of a row-contiguous tile, one per k-step of a k-contiguous tile) + a compile-time
   // offset (stage, k-step, fragment row block) that goes into the instruction's 16-bit offset field;
   // what does not fit the field is added to the base in units of 64 KiB.
   const unsigned lds0 = (unsigned)(unsigned long)lds_all;
-  // row-contiguous tile (nch chunks per row at byte offset toff of a stage): a lane reads 8 k values of
-  // column rowbase + lane%MF, k = kb .. kb+7 with kb = s*KS + 8*fgrp, from two 4(k) x 16(n) blocks.
-  // The swizzle of row k depends on the lane only (k&3 = (tx/4)&3, (k>>3)&1 = fgrp&1: KS is a multiple of 16).
-  auto tr_lane_base = [&](int toff, int nch, int rowbase) {
-    const int n = rowbase + 16 * tsub + 4 * (tx % 4);
-    const int k = 8 * fgrp + tx / 4;
-    return lds0 + (unsigned)(toff + (k * nch + ((n / 8) ^ swz_n(k, nch))) * 16 + (n % 8) * 2);
+  // Row-contiguous tile (nch chunks per row at byte offset toff of a stage): a lane reads the G k values
+  // kb .. kb+G-1, kb = s*KS + G*fgrp, of column rowbase + lane%MF.
+  //   16-bit: from two 4(k) x 16(n) blocks, each with one transposing read (16 lanes read a block and
+  //           each receives a column);
+  //   32-bit: one 32-bit read per k value.
+  // The swizzle of a row depends on the lane only (swz_n looks at k bits that s and the read number do
+  // not change).
+  auto rc_lane_base = [&](int toff, int nch, int rowbase) {
+    if constexpr (ES == 2) {
+      const int n = rowbase + 16 * tsub + 4 * (tx % 4);
+      const int k = 8 * fgrp + tx / 4;
+      return lds0 + (unsigned)(toff + (k * nch + ((n / 8) ^ swz_n(k, nch))) * 16 + (n % 8) * 2);
+    } else {
+      const int n = rowbase + frow;
+      const int k = 4 * fgrp;
+      return lds0 + (unsigned)(toff + (k * nch + ((n / 4) ^ swz_n(k, nch))) * 16 + (n % 4) * 4);
+    }
   };
   unsigned b_lane[TNI];
 #pragma unroll
-  for (int j = 0; j < TNI; ++j) b_lane[j] = tr_lane_base(A_BYTES, NCHB, wx * WN + j * MF);
+  for (int j = 0; j < TNI; ++j) b_lane[j] = rc_lane_base(A_BYTES, NCHB, wx * WN + j * MF);
   constexpr int NALANE = AK ? SPW : TMI;
   unsigned a_lane[NALANE];
   if constexpr (AK) {
@@ -764,15 +807,25 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       a_lane[st] = lds0 + (unsigned)(LK::slot(wy * WM + frow, st * KH + fgrp) * 16);   // swizzle: row%16 = frow%16 only
   } else {
 #pragma unroll
-    for (int i = 0; i < TMI; ++i) a_lane[i] = tr_lane_base(0, NCHA, wy * WM + i * MF);
+    for (int i = 0; i < TMI; ++i) a_lane[i] = rc_lane_base(0, NCHA, wy * WM + i * MF);
   }
   auto split_base = [](unsigned lane_base, int imm) { return lane_base + (unsigned)(imm / 65536) * 65536u; };
-  auto read_tr = [&](unsigned lane_base, auto imm_c, auto nch_c, FragTr* dst) {
-    constexpr int IMM0 = decltype(imm_c)::value;
-    constexpr int IMM1 = IMM0 + 4 * decltype(nch_c)::value * 16;      // second block: four rows further
-    const unsigned base0 = split_base(lane_base, IMM0), base1 = split_base(lane_base, IMM1);
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[0]) : "v"(base0), "n"(IMM0 % 65536));
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[1]) : "v"(base1), "n"(IMM1 % 65536));
+  auto read_rc = [&](unsigned lane_base, auto imm_c, auto nch_c, FragRc* dst) {
+    constexpr int IMM0 = decltype(imm_c)::value, ROW = decltype(nch_c)::value * 16;   // bytes per tile row
+    if constexpr (ES == 2) {
+      constexpr int IMM1 = IMM0 + 4 * ROW;                              // second block: four rows further
+      const unsigned base0 = split_base(lane_base, IMM0), base1 = split_base(lane_base, IMM1);
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[0]) : "v"(base0), "n"(IMM0 % 65536));
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[1]) : "v"(base1), "n"(IMM1 % 65536));
+    } else {
+      constexpr int IMM1 = IMM0 + ROW, IMM2 = IMM0 + 2 * ROW, IMM3 = IMM0 + 3 * ROW;   // one tile row per k value
+      const unsigned base0 = split_base(lane_base, IMM0), base1 = split_base(lane_base, IMM1);
+      const unsigned base2 = split_base(lane_base, IMM2), base3 = split_base(lane_base, IMM3);
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[0]) : "v"(base0), "n"(IMM0 % 65536));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[1]) : "v"(base1), "n"(IMM1 % 65536));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[2]) : "v"(base2), "n"(IMM2 % 65536));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[3]) : "v"(base3), "n"(IMM3 % 65536));
+    }
   };
   // fragment f of k-step s of the stage: s, f and the stage are compile-time constants (IntC)
   auto load_a = [&](auto stage_c, auto s_c, auto f_c, FragA* dst) {
@@ -782,12 +835,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       const unsigned base = split_base(a_lane[S], IMM);
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst->q) : "v"(base), "n"(IMM % 65536));
     } else {
-      read_tr(a_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHA * 16>(), IntC<NCHA>(), dst);
+      read_rc(a_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHA * 16>(), IntC<NCHA>(), dst);
     }
   };
   auto load_b = [&](auto stage_c, auto s_c, auto f_c, FragB* dst) {
     constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
-    read_tr(b_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHB * 16>(), IntC<NCHB>(), dst);
+    read_rc(b_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHB * 16>(), IntC<NCHB>(), dst);
   };
   // lgkmcnt(0): every LDS read issued so far has returned
   auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
@@ -826,7 +879,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // (the further ahead, the earlier the barrier stands in the last step and the more room the fetches
   // behind it have; measured best at the maximum)
   constexpr int DA = cmax(1, cmin(TMI - 1, KCG_SCHED_A_AHEAD > 0 ? KCG_SCHED_A_AHEAD : TMI - 1));
-  typedef StreamPlan<TMI, TNI, DA, (AK ? 1 : 2), 2> SP;
+  typedef StreamPlan<TMI, TNI, DA, (AK ? 1 : RC_READS), RC_READS> SP;
   constexpr int RB = SP::RB;
   constexpr int MT = SPW * NM;
   constexpr int BAR = (SPW - 1) * NM + RB * TNI;

@@ -63,6 +63,22 @@ EXACT_CASES = [
     ("mfma-odd-at1", MFMA, dict(M=131, N=67, K=37, is_atrans=1, lsu=2, BK=32)),
     ("mfma-64x48", MFMA, dict(M=256, N=192, K=128, BM=64, BN=48, BK=32, TM=4, TN=6, scatter=2, glw=2, gsw=2, lsu=2)),
     ("simt-64x48", SIMT, dict(M=256, N=192, K=128, BM=64, BN=48, BK=32, TM=4, TN=6, scatter=2, glw=2, gsw=2, lsu=2)),
+    # fp32 through the direct-staging kernel (both prefetch flags + LOAD_CONTINUOUS): 4, 2 and 3 LDS stages,
+    # both A layouts, long K (steady-state loop), 32x32 and 16x16 matrix-core tiles, 8 waves
+    ("f32-direct-128-at0", MFMA, dict(M=256, N=256, K=256, BM=128, BN=128, TM=8, TN=8, BK=16, is_atrans=0,
+                                      shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-128-at1-longk", MFMA, dict(M=256, N=256, K=1040, BM=128, BN=128, TM=8, TN=8, BK=16, is_atrans=1,
+                                            shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-256-2st", MFMA, dict(M=256, N=512, K=1024, BM=256, BN=256, TM=16, TN=16, BK=32, is_atrans=0,
+                                      shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-256x128-3st-at1", MFMA, dict(M=512, N=256, K=1056, BM=256, BN=128, TM=16, TN=8, BK=32, is_atrans=1,
+                                              shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-bk8", MFMA, dict(M=256, N=256, K=520, BM=128, BN=128, TM=8, TN=8, BK=8, is_atrans=0,
+                                  shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-mf16-8w", MFMA, dict(M=256, N=256, K=544, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=0,
+                                      shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-mf16-8w-at1", MFMA, dict(M=256, N=256, K=544, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=1,
+                                          shared_prefetch=1, reg_prefetch=1)),
     ("mfma-bm0", MFMA, dict(M=512, N=256, K=64, block_mapping=0)),
     ("mfma-bm4", MFMA, dict(M=512, N=384, K=64, block_mapping=4)),
 ]
