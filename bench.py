@@ -33,6 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # by what the same counter read for a 256 MiB copy (FETCH x2.000, WRITE x1.000).  Keyed by the tile part
 # of the kernel name; a kernel that was not profiled reports null.
 MEASURED_TRAFFIC_BYTES = {
+    "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x8_BTmnk256x256x32_BLmn2x4": (2 * 196730 + 65569) * 1024,
     "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x16_BTmnk256x256x32_BLmn2x2": (2 * 196749 + 65536) * 1024,
     "DTabcfloat16xfloat16xfloat32_AT0_TTmn16x16_BTmnk256x256x64_BLmn2x2": (2 * 98428 + 65536) * 1024,
 }
