@@ -623,7 +623,12 @@ struct DirectPlan {
   // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
   static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * ES;
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
-  static constexpr int NST_CAP = NST_FIT < 2 ? 2 : (NST_FIT > 4 ? 4 : NST_FIT);
+  // and no more than the fetch counter can tell apart: the wait for tile kt+1 allows the fetches of
+  // NST-2 younger tiles in flight, and that counter has 6 bits
+  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
+  static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
+  static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
+  static constexpr int NST_CAP = NST_MAX < 2 ? 2 : (NST_MAX > 4 ? 4 : NST_MAX);
   static constexpr int NST = (SPW % 2 == 1 && NST_CAP % 2 == 1) ? NST_CAP - 1 : NST_CAP;
   // the host picks the path (it must size dynamic LDS accordingly); both sides have to agree
   static_assert(ELIGIBLE == C::DIRECT, "host and device disagree on the direct-staging eligibility rule");

@@ -79,6 +79,8 @@ EXACT_CASES = [
                                       shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-mf16-8w-at1", MFMA, dict(M=256, N=256, K=544, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=1,
                                           shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-1wave", MFMA, dict(M=256, N=256, K=1056, BM=128, BN=128, TM=16, TN=16, BK=32, is_atrans=0,
+                                    shared_prefetch=1, reg_prefetch=1)),
     ("mfma-bm0", MFMA, dict(M=512, N=256, K=64, block_mapping=0)),
     ("mfma-bm4", MFMA, dict(M=512, N=384, K=64, block_mapping=4)),
 ]
@@ -136,6 +138,9 @@ HALF_CASES = [
                               BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-2rows-at1", dict(M=192, N=128, K=736, dtype=2, dtype_c=4, is_atrans=1, BM=64, BN=64, TM=4, TN=4,
                                   BK=32, shared_prefetch=1, reg_prefetch=1)),
+    # one wave per block: 32 fetch instructions per wave and tile limit the number of stages in flight
+    ("f16-direct-1wave", dict(M=256, N=256, K=1088, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=16, TN=16,
+                              BK=64, shared_prefetch=1, reg_prefetch=1)),
     ("bf16-at0", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=0, BK=32)),
     ("bf16-at1-lsu2", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=1, BK=64, lsu=2)),
 ]
