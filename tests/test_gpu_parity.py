@@ -175,6 +175,9 @@ def extra_build_configs():
         out.append((make_config(4096, 1536, 1000, **kw), kind))
     for kw in CONFIG5_KERNELS:
         out.append((make_config(4096, 4096, 4096, dtype=2, dtype_c=4, is_atrans=0, **kw), MFMA))
+    bf16 = dict(_tuned("gemm_4096_fp16.json"))
+    bf16["DATATYPE_A"] = bf16["DATATYPE_B"] = 3
+    out.append((bf16, 0))
     return out
 
 
@@ -246,3 +249,31 @@ def test_config5_fp16_4096(oracle):
         lhs = got.astype(np.float64).sum(axis=0)
         rhs = a.astype(np.float64).sum(axis=0) @ b.astype(np.float64)
         assert np.abs(lhs - rhs).max() <= 2e-2 * scale * np.sqrt(M)
+
+
+def _tuned(name):
+    import json
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "codegendemo_amd", "TunedConfigs", name)) as f:
+        return json.load(f)["cfgs"][0]
+
+
+@pytest.mark.parametrize("which", ["fp32", "fp16", "bf16"])
+def test_tuned_4096_kernels_are_bit_exact_on_integers(oracle, which):
+    """The kernels bench.py launches (all 256 CUs busy, every stage of the K loop under real memory
+    latency), on integers in [-2, 2]: sums of 4096 products (<= 16384) are exact in fp32, so the whole
+    4096 x 4096 result must equal the oracle bit for bit whatever the summation order."""
+    cfg = dict(_tuned("gemm_4096_fp32.json" if which == "fp32" else "gemm_4096_fp16.json"))
+    if which == "bf16":
+        cfg["DATATYPE_A"] = cfg["DATATYPE_B"] = 3
+    M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+    a = SI.small_ints((M, K), SI.STREAM_A, lim=2)
+    b = SI.small_ints((K, N), SI.STREAM_B, lim=2)
+    print(f"[case] tuned {which} {M}x{N}x{K}", flush=True)
+    got, info = run_gemm(cfg, a, b)
+    assert info["lds_bytes"] == 0          # the direct-staging kernel
+    want = oracle.matmul(a, b, a_trans=False)
+    assert not np.isnan(got).any()
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, f"tuned {which}: {len(bad)} mismatches, first at {bad[:5].tolist()}"
