@@ -147,12 +147,12 @@ MfmaPlan plan_mfma(const MatmulConfig& c) {
     p.why = "wave tile (WARP_LAYOUT*THREAD_SIZE) is not a multiple of the 16x16 matrix-core tile";
     return p;
   }
-  p.MF = (p.WM % 32 == 0 && p.WN % 32 == 0) ? 32 : 16;
   const int sz = dtype_size(c.dtA);
-  if (sz != 2 && sz != 4) {
-    p.why = "matrix-core kernel supports float32, float16 and bfloat16 inputs";
+  if (sz != 2 && sz != 4 && sz != 8) {
+    p.why = "matrix-core kernel supports float64, float32, float16 and bfloat16 inputs";
     return p;
   }
+  p.MF = (sz != 8 && p.WM % 32 == 0 && p.WN % 32 == 0) ? 32 : 16;   // fp64: 16x16x4 only
   p.G = 16 / sz;
   p.KS = p.G * (64 / p.MF);
   p.ok = true;
@@ -170,7 +170,8 @@ std::string check_mfma(const MatmulConfig& c) {
       << " matrix-core tile";
     return s.str();
   }
-  if ((p.WM / p.MF) * (p.WN / p.MF) * (p.MF * p.MF / 64) > 256) return "wave tile needs more than 256 accumulator registers";
+  if ((p.WM / p.MF) * (p.WN / p.MF) * (p.MF * p.MF / 64) * (dtype_size(c.dtA) == 8 ? 2 : 1) > 256)
+    return "wave tile needs more than 256 accumulator registers";
   if (c.LSU > 1 && (c.BN % c.GSW)) return "BLOCK_SIZE_N not divisible by GLOB_STORE_WIDTH";
   if (lds_bytes(c, KCG_KIND_MFMA) > kMaxLdsBytes) return "LDS footprint exceeds 160 KiB";
   if ((c.SHMP ? 2 : 1) * (c.BM + c.BN) * c.BK * dtype_size(c.dtA) > kMaxLdsBytes) return "LDS footprint exceeds 160 KiB";

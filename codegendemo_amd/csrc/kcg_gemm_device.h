@@ -29,6 +29,8 @@ namespace kcg {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef double doublex2 __attribute__((ext_vector_type(2)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
 typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -470,6 +472,16 @@ template <> struct Mfma<float, 16> {
   __device__ __forceinline__ static void run_tied(Acc& c, const Frag& a, const Frag& b) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+a"(c) : "v"(a[t]), "v"(b[t]));
+  }
+};
+// fp64: one instruction shape, 16x16x4 (lane: row/column lane%16, k = lane/16); a 16-byte chunk holds two
+// consecutive k values, so a fragment step is two instructions
+template <> struct Mfma<double, 16> {
+  typedef doublex4 Acc;
+  typedef doublex2 Frag;
+  __device__ __forceinline__ static void run(Acc& c, const Frag& a, const Frag& b) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) c = __builtin_amdgcn_mfma_f64_16x16x4f64(a[t], b[t], c, 0, 0, 0);
   }
 };
 template <> struct Mfma<_Float16, 32> {
@@ -1048,7 +1060,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
   constexpr int ES = (int)sizeof(T);
   constexpr int G = 16 / ES;                  // k elements per 16-byte chunk
   constexpr int WM = BM / C::BLM, WN = BN / C::BLN;   // wave tile = (WLM*TM) x (WLN*TN)
-  constexpr int MF = (WM % 32 == 0 && WN % 32 == 0) ? 32 : 16;
+  constexpr int MF = (ES != 8 && WM % 32 == 0 && WN % 32 == 0) ? 32 : 16;   // fp64 has the 16x16 shape only
   constexpr int KH = 64 / MF;                 // lane groups along k inside one instruction
   constexpr int KS = G * KH;                  // k covered by one fragment step
   constexpr int NSS = BK / KS;                // fragment steps per K tile
@@ -1062,6 +1074,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
   typedef Mfma<T, MF> MI;
   typedef typename MI::Acc Acc;
   typedef typename MI::Frag Frag;
+  typedef typename AccOf<T>::type AccT;       // float, or double for fp64 inputs
   typedef LdsTile<CH> L;
 
   u32x4* smA = reinterpret_cast<u32x4*>(smem);               // [STAGES][BM*CH] chunks
@@ -1161,7 +1174,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
 #pragma unroll
     for (int j = 0; j < TNI; ++j)
 #pragma unroll
-      for (int e = 0; e < (int)(sizeof(Acc) / sizeof(float)); ++e) acc[i][j][e] = 0.0f;
+      for (int e = 0; e < (int)(sizeof(Acc) / sizeof(AccT)); ++e) acc[i][j][e] = (AccT)0;
 
   const int frow = lane % MF;   // row of the MFMA tile this lane feeds
   const int fgrp = lane / MF;   // lane group along k
@@ -1300,12 +1313,14 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
 
   // ---- epilogue -------------------------------------------------------------------------------
   // Accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(e/4) + 4*(lane/32) + e%4
-  // for e in 0..15; of a 16x16 tile: column lane%16, rows 4*(lane/16) + e for e in 0..3.
-  constexpr int NACC = (int)(sizeof(Acc) / sizeof(float));
+  // for e in 0..15; of a 16x16 tile: column lane%16, rows 4*(lane/16) + e for e in 0..3; of the fp64
+  // 16x16 tile: column lane%16, rows lane/16 + 4*e (established on hardware; the parity tests pin it).
+  constexpr int NACC = (int)(sizeof(Acc) / sizeof(AccT));
   const int ocol = lane % MF;
   const int orow = (lane / MF) * 4;
+  auto acc_row = [&](int e) { return ES == 8 ? lane / MF + 4 * e : (e / 4) * 8 + orow + e % 4; };
   if constexpr (LSU > 1) {
-    float* smC = reinterpret_cast<float*>(smem);
+    AccT* smC = reinterpret_cast<AccT*>(smem);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < TMI; ++i)
@@ -1313,7 +1328,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
       for (int j = 0; j < TNI; ++j)
 #pragma unroll
         for (int e = 0; e < NACC; ++e) {
-          const int row = wy * WM + i * MF + (e / 4) * 8 + orow + e % 4;
+          const int row = wy * WM + i * MF + acc_row(e);
           const int col = wx * WN + j * MF + ocol;
           smC[(wz * BM + row) * BN + col] = acc[i][j][e];
         }
@@ -1326,7 +1341,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
       for (int j = 0; j < TNI; ++j)
 #pragma unroll
         for (int e = 0; e < NACC; ++e) {
-          const int row = m0 + wy * WM + i * MF + (e / 4) * 8 + orow + e % 4;
+          const int row = m0 + wy * WM + i * MF + acc_row(e);
           const int col = n0 + wx * WN + j * MF + ocol;
           if (!EDGE || (row < M && col < N)) Cm[(long)row * N + col] = (TC)acc[i][j][e];
         }

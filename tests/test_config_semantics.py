@@ -154,7 +154,9 @@ def test_kind_selection_rules():
     assert _native.select_kind(v) == _native.KIND_SIMT
     v = vals(make_config(1024, 1024, 1024, BM=64, BN=48, BK=32, TM=4, TN=6, scatter=2, glw=2, gsw=2))  # 32x48 wave tile
     assert _native.select_kind(v) == _native.KIND_MFMA                      # 32x48 wave tile = 2x3 tiles of 16x16
-    v = vals(make_config(512, 512, 512, dtype=8, BM=64, BN=64, BK=16, glw=2, gsw=2, scatter=2))         # fp64: SIMT only
+    v = vals(make_config(512, 512, 512, dtype=8, BM=64, BN=64, BK=16, glw=2, gsw=2, scatter=2))         # fp64: 16x16x4 tiles, BK%8
+    assert _native.select_kind(v) == _native.KIND_MFMA
+    v = vals(make_config(512, 512, 512, dtype=8, BM=64, BN=64, BK=4, glw=2, gsw=2, scatter=2))          # fp64 with BK=4: SIMT
     assert _native.select_kind(v) == _native.KIND_SIMT
 
 

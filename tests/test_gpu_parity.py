@@ -44,6 +44,9 @@ EXACT_CASES = [
     ("simt-edge", SIMT, dict(M=200, N=136, K=100)),
     ("simt-edge-at0", SIMT, dict(M=200, N=136, K=100, is_atrans=0, shared_prefetch=1)),
     ("simt-odd", SIMT, dict(M=131, N=67, K=37, is_atrans=0, lsu=2)),
+    ("simt-f64", SIMT, dict(M=256, N=256, K=128, dtype=8, scatter=2)),
+    ("simt-f64-at0-both", SIMT, dict(M=256, N=192, K=136, dtype=8, scatter=2, is_atrans=0, shared_prefetch=1, reg_prefetch=1, BK=8)),
+    ("simt-f64-lsu2-edge", SIMT, dict(M=200, N=136, K=100, dtype=8, scatter=1, lsu=2)),
     ("mfma-base", MFMA, dict(M=256, N=256, K=128)),
     ("mfma-atrans0", MFMA, dict(M=256, N=256, K=128, is_atrans=0)),
     ("mfma-shmp", MFMA, dict(M=256, N=256, K=128, shared_prefetch=1)),
@@ -81,6 +84,13 @@ EXACT_CASES = [
                                           shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-1wave", MFMA, dict(M=256, N=256, K=1056, BM=128, BN=128, TM=16, TN=16, BK=32, is_atrans=0,
                                     shared_prefetch=1, reg_prefetch=1)),
+    # fp64 on the matrix cores (16x16x4 instructions, two k values per 16-byte chunk)
+    ("mfma-f64", MFMA, dict(M=256, N=256, K=128, dtype=8, scatter=2)),
+    ("mfma-f64-at0-both", MFMA, dict(M=256, N=192, K=136, dtype=8, scatter=2, is_atrans=0, shared_prefetch=1,
+                                     reg_prefetch=1, BK=8)),
+    ("mfma-f64-128x128", MFMA, dict(M=256, N=256, K=256, dtype=8, scatter=2, BM=128, BN=128, TM=8, TN=8, BK=16,
+                                    is_atrans=0, shared_prefetch=1, reg_prefetch=1)),
+    ("mfma-f64-lsu2-edge", MFMA, dict(M=200, N=136, K=100, dtype=8, scatter=1, lsu=2)),
     ("mfma-bm0", MFMA, dict(M=512, N=256, K=64, block_mapping=0)),
     ("mfma-bm4", MFMA, dict(M=512, N=384, K=64, block_mapping=4)),
 ]
