@@ -101,6 +101,24 @@ def time_steps(kernel, A, B, C, steps, warmup):
     return (t1 - t0) * 1e3 / steps, ev0.elapsed_time(ev1) / steps
 
 
+def time_library_gemm(A, B, a_trans, steps, warmup):
+    """The vendor library's GEMM (torch.matmul -> rocBLAS/hipBLASLt) on the same device buffers, timed like
+    time_steps: for orientation only, it is neither the oracle nor part of the product."""
+    import torch
+    a = A.t() if a_trans else A
+    for _ in range(warmup):
+        torch.matmul(a, B)
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(steps):
+        torch.matmul(a, B)
+    ev1.record()
+    torch.cuda.synchronize()
+    return ev0.elapsed_time(ev1) / steps
+
+
 def cpu_baseline(a, b, ijk_seconds=8.0):
     """Times the CPU oracle on this box's host cores: the threaded loop over the WHOLE 4096^3 product
     (best of 3; it is also the parity reference for the GPU result) and, for the record, the
@@ -191,6 +209,7 @@ def main():
     value = flops / (ms_step * 1e-3) / 1e12
     achieved = flops / (ms_launch * 1e-3) / 1e12
     c_host = C.cpu().numpy()
+    lib_ms = time_library_gemm(A, B, kpm.isATranspose, args.steps, args.warmup)
 
     out = {
         "metric": "GEMM TFLOPS and % of dtype MFMA roofline at M=N=K=4096, 1 MI355X",
@@ -206,12 +225,16 @@ def main():
                      "hbm_gbs_algorithmic": (4.0 * (kpm.M * kpm.K + kpm.K * kpm.N + kpm.M * kpm.N)) / (ms_launch * 1e-3) / 1e9},
     }
 
+    out["library_gemm"] = {"source": "torch.matmul (rocBLAS/hipBLASLt) on the same buffers, same timing loop",
+                           "f32_tflops": flops / (lib_ms * 1e-3) / 1e12}
     if not args.no_fp16:
         cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
         kpm16, kernel16, info16 = build_kernel(cfg16)
         _, _, A16, B16, C16 = make_inputs(kpm16, "normal")
         ms_step16, ms_launch16 = time_steps(kernel16, A16, B16, C16, args.steps, args.warmup)
         ach16 = flops / (ms_launch16 * 1e-3) / 1e12
+        lib16_ms = time_library_gemm(A16, B16, kpm16.isATranspose, args.steps, args.warmup)
+        out["library_gemm"]["f16_tflops"] = flops / (lib16_ms * 1e-3) / 1e12
         out["fp16"] = {"value": flops / (ms_step16 * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_step16,
                        "dtype": "f16 in, f32 accumulate/out", "kernel": info16["kernel_name"],
                        "roofline": {"bound": "mfma", "achieved": ach16, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
