@@ -27,15 +27,26 @@
 
 #define KCG_VERSION "kcg-gemm-gfx950 0.1"
 
-// The device template header, embedded at build time (path given by -DKCG_DEVICE_HEADER_PATH).
-__asm__(
-    ".section .rodata\n"
-    ".global kcg_device_src\n"
-    "kcg_device_src:\n"
-    ".incbin \"" KCG_DEVICE_HEADER_PATH "\"\n"
-    ".byte 0\n"
-    ".previous\n");
-extern "C" const char kcg_device_src[];
+// The device template headers, embedded at build time (directory given by -DKCG_DEVICE_HEADER_DIR):
+// kcg_gemm_device.h is what the instantiation stub includes; it includes the others.
+#define KCG_EMBED(sym, file)                         \
+  __asm__(".section .rodata\n"                       \
+          ".global " #sym "\n" #sym ":\n"            \
+          ".incbin \"" KCG_DEVICE_HEADER_DIR "/" file "\"\n" \
+          ".byte 0\n"                                \
+          ".previous\n");                            \
+  extern "C" const char sym[];
+KCG_EMBED(kcg_device_src, "kcg_gemm_device.h")
+KCG_EMBED(kcg_device_src_common, "kcg_device_common.h")
+KCG_EMBED(kcg_device_src_simt, "kcg_device_simt.h")
+KCG_EMBED(kcg_device_src_mfma_ops, "kcg_device_mfma_ops.h")
+KCG_EMBED(kcg_device_src_direct, "kcg_device_direct.h")
+KCG_EMBED(kcg_device_src_mfma, "kcg_device_mfma.h")
+static const char* const kDeviceHeaderNames[] = {"kcg_gemm_device.h",     "kcg_device_common.h", "kcg_device_simt.h",
+                                                 "kcg_device_mfma_ops.h", "kcg_device_direct.h", "kcg_device_mfma.h"};
+static const char* const kDeviceHeaderSrcs[] = {kcg_device_src,          kcg_device_src_common, kcg_device_src_simt,
+                                                kcg_device_src_mfma_ops, kcg_device_src_direct, kcg_device_src_mfma};
+static const int kNumDeviceHeaders = 6;
 
 namespace {
 
@@ -435,7 +446,7 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   h = fnv1a(arch, h);
   h = fnv1a(flags_text, h);
   h = fnv1a(stub, h);
-  h = fnv1a(kcg_device_src, h);
+  for (int i = 0; i < kNumDeviceHeaders; ++i) h = fnv1a(kDeviceHeaderSrcs[i], h);
   char hex[32];
   snprintf(hex, sizeof(hex), "%016llx", (unsigned long long)h);
 
@@ -452,9 +463,9 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   }
 
   hiprtcProgram prog;
-  const char* hdr_src[] = {kcg_device_src};
-  const char* hdr_name[] = {"kcg_gemm_device.h"};
-  hiprtcResult r = RTCF(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", 1, hdr_src, hdr_name);
+  hiprtcResult r = RTCF(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", kNumDeviceHeaders,
+                                             const_cast<const char**>(kDeviceHeaderSrcs),
+                                             const_cast<const char**>(kDeviceHeaderNames));
   if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTCF(hiprtcGetErrorString)(r));
   std::vector<std::string> opts = compile_flags();
   opts.push_back("--offload-arch=" + arch);

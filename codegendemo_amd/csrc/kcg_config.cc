@@ -215,7 +215,7 @@ int reference_lds_bytes(const MatmulConfig& c) {
 }
 
 // (That kernel keeps 2..4 stages of (BM+BN)*BK*2 bytes in static LDS: as many as fit in 160 KiB.)
-// Must state the same rule as DirectPlan<C>::ELIGIBLE in kcg_gemm_device.h (a static_assert there
+// Must state the same rule as DirectPlan<C>::ELIGIBLE in kcg_device_direct.h (a static_assert there
 // compares the two): 16-bit inputs or fp32 throughout, no edge tiles, both prefetch flags, LOAD_CONTINUOUS, 128-bit load
 // widths, power-of-two tiles that split evenly into 1 KiB wave fetches, at least two rows of
 // matrix-core tiles per wave, and two LDS stages within 160 KiB.

@@ -1,0 +1,203 @@
+// kcg_device_common.h — vector types, compile-time helpers, block scheduling, global load/store helpers
+// and the split-U reduce shared by all kernel families of kcg_gemm_device.h.
+#pragma once
+
+namespace kcg {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef double doublex2 __attribute__((ext_vector_type(2)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int BYTES> struct RawVec;
+template <> struct RawVec<1> { typedef unsigned char type; };
+template <> struct RawVec<2> { typedef unsigned short type; };
+template <> struct RawVec<4> { typedef unsigned int type; };
+template <> struct RawVec<8> { typedef u32x2 type; };
+template <> struct RawVec<16> { typedef u32x4 type; };
+
+template <class T> struct AccOf { typedef float type; };
+template <> struct AccOf<double> { typedef double type; };
+
+constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
+constexpr int cmin(int a, int b) { return a < b ? a : b; }
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+constexpr int lowbit(int a) { return a & (-a); }
+template <bool B> struct BoolC { static constexpr bool value = B; };
+template <bool B, class X, class Y> struct Select { typedef X type; };
+template <class X, class Y> struct Select<false, X, Y> { typedef Y type; };
+template <int I> struct IntC { static constexpr int value = I; };
+// f(IntC<Begin>()), ..., f(IntC<End-1>()) — a loop whose index is a compile-time constant in the body
+template <int Begin, int End, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (Begin < End) {
+    f(IntC<Begin>());
+    static_for<Begin + 1, End>(f);
+  }
+}
+
+// Copy NBYTES (power of two, <= 16) between two suitably aligned addresses as one access.
+template <int NBYTES>
+__device__ __forceinline__ void copy_bytes(void* dst, const void* src) {
+  typedef typename RawVec<NBYTES>::type V;
+  *reinterpret_cast<V*>(dst) = *reinterpret_cast<const V*>(src);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Block id -> (by, bx).  Rewriter::BlockMapping (Rewriter.cc:726-761): groups of BLOCK_MAPPING block
+// rows are walked column by column so that concurrently resident blocks share B panels in L2.
+// On top of it, when the block count is a multiple of 8, consecutive hardware ids (which the
+// dispatcher deals round-robin to the 8 XCDs, each with a private L2) are remapped so that every XCD
+// walks one contiguous eighth of that order.
+// ---------------------------------------------------------------------------------------------
+template <class C>
+__device__ __forceinline__ void block_coords(int bid, int& by, int& bx) {
+  constexpr int GY = cdiv(C::M, C::BM);
+  constexpr int GX = cdiv(C::N, C::BN);
+  constexpr int NB = GY * GX;
+  if constexpr (C::XCD_REMAP && (NB % 8 == 0)) {
+    bid = (bid % 8) * (NB / 8) + bid / 8;
+  }
+  if constexpr (C::BLOCK_MAPPING > 0 && (GY % (C::BLOCK_MAPPING > 0 ? C::BLOCK_MAPPING : 1) == 0)) {
+    constexpr int G = C::BLOCK_MAPPING;
+    constexpr int GN = G * GX;
+    by = (bid / GN) * G + bid % G;
+    bx = (bid % GN) / G;
+  } else {
+    by = bid / GX;
+    bx = bid % GX;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Thread -> vector map over a ROWS x COLS tile whose COLS dimension is contiguous in memory.
+//   CONT=1 ("LOAD_CONTINUOUS", Optimizer.cc:79-83):  v = tid + it*NT, row = v / VPR, col = (v % VPR)*VEC
+//   CONT=0 (Optimizer.cc:84-88): row = tid / (NT/ROWS), col = it*(NT/ROWS*VEC) + (tid % (NT/ROWS))*VEC
+// ---------------------------------------------------------------------------------------------
+template <int ROWS, int COLS, int VEC, int NT, bool CONT>
+struct TileMap {
+  static constexpr int VPR = COLS / VEC;
+  static constexpr int NV = ROWS * VPR;
+  static constexpr int TPR = CONT ? 1 : NT / ROWS;
+  static constexpr int ITERS = CONT ? cdiv(NV, NT) : COLS / (TPR * VEC);
+  static constexpr bool FULL = CONT ? (NV % NT == 0) : true;
+  __device__ __forceinline__ static bool coords(int tid, int it, int& r, int& c) {
+    if constexpr (CONT) {
+      int v = tid + it * NT;
+      r = v / VPR;
+      c = (v % VPR) * VEC;
+      return FULL || v < NV;
+    } else {
+      r = tid / TPR;
+      c = it * (TPR * VEC) + (tid % TPR) * VEC;
+      return true;
+    }
+  }
+};
+
+// Thread -> (k chunk, first row) map for an operand tile that is contiguous along m/n in global memory
+// and is transposed into [row][k chunk] LDS layout: NCH k-chunks x NVEC row vectors of VEC rows.
+//   ROWS_FAST=1: consecutive threads take consecutive row vectors (widest global coalescing)
+//   ROWS_FAST=0: consecutive threads take consecutive k chunks of one row vector, so the 16-byte LDS
+//                writes of 8 neighbouring lanes land in 8 different bank groups
+template <int NCH, int NVEC, int VEC, int NT, bool ROWS_FAST>
+struct BlockMap {
+  static constexpr int NB = NCH * NVEC;
+  static constexpr int ITERS = cdiv(NB, NT);
+  static constexpr bool FULL = (NB % NT == 0);
+  __device__ __forceinline__ static bool coords(int tid, int it, int& chunk, int& row) {
+    int v = tid + it * NT;
+    if constexpr (ROWS_FAST) {
+      chunk = v / NVEC;
+      row = (v % NVEC) * VEC;
+    } else {
+      chunk = v % NCH;
+      row = (v / NCH) * VEC;
+    }
+    return FULL || v < NB;
+  }
+};
+
+// Load VEC consecutive elements T from row r, column c of a row-major matrix with leading dimension
+// LD into dst[0..VEC).  With EDGE, elements outside [0,RMAX) x [0,CMAX) read as zero.  ALIGNED says
+// every such vector is naturally aligned to VEC*sizeof(T) so one wide load is legal.
+template <class T, int VEC, bool EDGE, bool ALIGNED>
+__device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r, int c, int LD, int RMAX, int CMAX) {
+  if constexpr (!EDGE) {
+    if constexpr (ALIGNED) {
+      copy_bytes<VEC * (int)sizeof(T)>(dst, base + (long)r * LD + c);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) dst[e] = base[(long)r * LD + c + e];
+    }
+  } else {
+    if (ALIGNED && r < RMAX && c + VEC <= CMAX) {
+      copy_bytes<VEC * (int)sizeof(T)>(dst, base + (long)r * LD + c);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        dst[e] = (r < RMAX && c + e < CMAX) ? base[(long)r * LD + c + e] : T(0);
+      }
+    }
+  }
+}
+
+// Store VEC consecutive output elements (converted from the accumulator type) with the same rules.
+template <class TC, class ACC, int VEC, bool EDGE, bool ALIGNED>
+__device__ __forceinline__ void gstore(TC* __restrict__ base, const ACC* src, int r, int c, int LD, int RMAX, int CMAX) {
+  TC tmp[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) tmp[e] = (TC)src[e];
+  if constexpr (!EDGE) {
+    if constexpr (ALIGNED) {
+      copy_bytes<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) base[(long)r * LD + c + e] = tmp[e];
+    }
+  } else {
+    if (ALIGNED && r < RMAX && c + VEC <= CMAX) {
+      copy_bytes<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        if (r < RMAX && c + e < CMAX) base[(long)r * LD + c + e] = tmp[e];
+    }
+  }
+}
+
+// Split-U epilogue shared by both families (Rewriter::splitUReduce / splitUWrite, Rewriter.cc:603-663):
+// smC is [LSU][BM][BN] accumulators; slice 0 is copied, slices 1..LSU-1 are added in order, and the
+// sum is written to C with GLOB_STORE_WIDTH-wide vectors using the (non-)continuous map selected by
+// REDUCE_C_CONTINUOUS (Optimizer.cc:241-282).
+template <class C, int NT>
+__device__ __forceinline__ void splitu_reduce_store(typename C::TC* __restrict__ Cm, const typename C::ACC* smC,
+                                                    int tid, int m0, int n0) {
+  typedef typename C::ACC ACC;
+  constexpr int GSW = C::GSW;
+  constexpr bool CONT = C::RC != 0 || (NT % C::BM != 0) || (C::BN % ((NT / C::BM) * GSW) != 0);
+  typedef TileMap<C::BM, C::BN, GSW, NT, CONT> Map;
+  constexpr bool ALIGNED = (C::N % GSW == 0);
+#pragma unroll
+  for (int it = 0; it < Map::ITERS; ++it) {
+    int r, c;
+    if (Map::coords(tid, it, r, c)) {
+      ACC sum[GSW];
+#pragma unroll
+      for (int e = 0; e < GSW; ++e) sum[e] = smC[r * C::BN + c + e];
+#pragma unroll
+      for (int z = 1; z < C::LSU; ++z) {
+#pragma unroll
+        for (int e = 0; e < GSW; ++e) sum[e] += smC[(z * C::BM + r) * C::BN + c + e];
+      }
+      gstore<typename C::TC, ACC, GSW, C::EDGE, ALIGNED>(Cm, sum, m0 + r, n0 + c, C::N, C::M, C::N);
+    }
+  }
+}
+
+}  // namespace kcg

@@ -1,0 +1,502 @@
+// kcg_device_direct.h — kernel family 2b: matrix-core kernel with direct global->LDS staging and a
+// row-streaming, hand-scheduled K loop (fp32, fp16, bf16 inputs).
+#pragma once
+#include "kcg_device_common.h"
+#include "kcg_device_mfma_ops.h"
+
+namespace kcg {
+
+// =============================================================================================
+// Family 2b: matrix-core kernel with direct global->LDS staging (16-bit inputs).
+//
+// Every lane fetches one 16-byte chunk with global_load_lds_dwordx4; a wave's 64 chunks land in 1 KiB of
+// consecutive LDS, so no register, no ds_write and no VALU work is spent on staging and the fetch of
+// tile kt+2 can be in flight for a whole K tile.  The LDS image keeps the orientation of global memory:
+//   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/8 chunks of 8 k values each; a fragment
+//                                           is one ds_read_b128 (as in gemm_mfma)
+//   row-contiguous operand (B; A^T)       : rows = k, NCH = BN/8 (BM/8) chunks of 8 n values each; a
+//                                           fragment is two ds_read_b64_tr_b16: 16 lanes read a 4(k) x
+//                                           16(n) block and each lane receives one column of it, which
+//                                           is the k-packed layout the matrix core wants
+// The bank swizzle is applied on the fetch side: the lane that fills physical chunk c' of a row fetches
+// logical chunk c' ^ swz(row), and readers look chunk c up at c ^ swz(row).
+// =============================================================================================
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+// Static schedule of the fragment reads of one k-step of the direct-staging kernel (see its K loop):
+// which slot reads which B fragment of the next step, and how many LDS read instructions issued after
+// the fragments a row needs may still be in flight when that row starts.
+template <int TMI, int TNI, int DA, int NAI, int NBI>
+struct StreamPlan {
+  static constexpr int NM = TMI * TNI;
+  static constexpr int RB = TMI - DA;                              // first row whose side work belongs to the next step
+  static constexpr int BW0 = RB * TNI;                             // B reads: slots [BW0, BW1)
+  static constexpr int BW1 = DA > 1 ? (TMI - 1) * TNI : NM;
+  static constexpr int slot_b(int j) { return BW0 + (j * (BW1 - BW0)) / TNI; }
+  // issue times in half slots: a row's A read comes first in its slot, a B read follows the
+  // matrix-core instruction of its slot
+  static constexpr int time_a(int step, int row) { return (step * NM + (row - DA) * TNI) * 2; }
+  static constexpr int time_b(int step, int j) { return ((step - 1) * NM + slot_b(j)) * 2 + 1; }
+  static constexpr int allowed(int row) {
+    const int step = 2;
+    const int now = (step * NM + row * TNI) * 2 - 1;               // just before this row's own A read
+    int need = time_a(step, row);
+    if (row == 0)
+      for (int j = 0; j < TNI; ++j) need = cmax(need, time_b(step, j));
+    int n = 0;
+    for (int st = 0; st <= step + 1; ++st) {
+      for (int r = 0; r < TMI; ++r) {
+        const int t = time_a(st, r);
+        if (t > need && t < now) n += NAI;
+      }
+      for (int j = 0; j < TNI; ++j) {
+        const int t = time_b(st, j);
+        if (t > need && t < now) n += NBI;
+      }
+    }
+    return cmin(n, 15);                                            // the counter field has 4 bits; less is safe
+  }
+};
+
+template <class C>
+struct DirectPlan {
+  typedef typename C::TA T;
+  static constexpr int ES = (int)sizeof(T);
+  static constexpr int WM = C::BM / C::BLM, WN = C::BN / C::BLN;
+  // 16x16x32 instructions where the K tile allows: on fp16/bf16 data with realistic bit activity a
+  // gfx950 sustains about 16 % more flops with them than with 32x32x16 at its power limit
+#ifndef KCG_DIRECT_MF
+#define KCG_DIRECT_MF 0               /* 16 or 32 forces the matrix-core tile of the direct-staging kernel */
+#endif
+  static constexpr int G = 16 / ES;                               // elements per 16-byte chunk
+  static constexpr bool FITS32 = WM % 32 == 0 && WN % 32 == 0;
+  static constexpr int MF = KCG_DIRECT_MF ? KCG_DIRECT_MF
+                            : ES == 2 ? ((C::BK % 32 == 0 || !FITS32) ? 16 : 32)
+                                      : (FITS32 ? 32 : 16);       // fp32: no such difference, the larger tile reads less
+  static constexpr int KS = G * (64 / MF);                        // k per step: one chunk per lane
+  static constexpr int NW = C::BLM * C::BLN;
+  static constexpr int NM = (WM / MF) * (WN / MF);
+  static constexpr int SPW = (C::BK % KS == 0) ? C::BK / KS : 0;
+  static constexpr bool pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+  static constexpr bool ELIGIBLE =
+      (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && !C::EDGE && C::SHMP && C::REGP && C::LC != 0 &&
+      C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
+      SPW > 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
+      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
+      (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024;
+  // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles); an even number
+  // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
+  static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * ES;
+  static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
+  // and no more than the fetch counter can tell apart: the wait for tile kt+1 allows the fetches of
+  // NST-2 younger tiles in flight, and that counter has 6 bits
+  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
+  static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
+  static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
+  static constexpr int NST_CAP = NST_MAX < 2 ? 2 : (NST_MAX > 4 ? 4 : NST_MAX);
+  static constexpr int NST = (SPW % 2 == 1 && NST_CAP % 2 == 1) ? NST_CAP - 1 : NST_CAP;
+  // the host picks the path (it must size dynamic LDS accordingly); both sides have to agree
+  static_assert(ELIGIBLE == C::DIRECT, "host and device disagree on the direct-staging eligibility rule");
+  static constexpr bool OK = C::DIRECT;
+};
+
+template <class C>
+__device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
+                                                 typename C::TC* __restrict__ Cm, char* smem) {
+  typedef typename C::TA T;
+  typedef typename C::TC TC;
+  typedef DirectPlan<C> P;
+  constexpr int BM = C::BM, BN = C::BN, BK = C::BK;
+  constexpr int M = C::M, N = C::N, K = C::K;
+  constexpr int WM = P::WM, WN = P::WN, MF = P::MF;
+  constexpr int KH = 64 / MF, KS = P::KS, SPW = P::SPW;
+  constexpr int TMI = WM / MF, TNI = WN / MF, NM = P::NM, NW = P::NW;
+  constexpr int KT = K / BK;
+  constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
+  constexpr int ES = P::ES, G = P::G;                   // element size; elements per 16-byte chunk
+  constexpr int CHK = BK / G;                           // chunks per row of a k-contiguous tile
+  constexpr int NCHA = BM / G, NCHB = BN / G;           // chunks per row of a row-contiguous tile
+  constexpr int A_BYTES = BM * BK * ES, B_BYTES = BN * BK * ES, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int NIA = (BM * BK / G) / (64 * NW);        // fetch instructions per wave and tile, operand A
+  constexpr int NIB = (BN * BK / G) / (64 * NW);
+  typedef Mfma<T, MF> MI;
+  typedef typename MI::Acc Acc;
+  typedef typename MI::Frag Frag;
+  typedef LdsTile<CHK> LK;
+
+  const int tid = threadIdx.x;
+  // the wave number is the same in all lanes: saying so keeps everything derived from it (LDS fetch
+  // destinations, which go through M0, and the wave's tile origin) in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int wy = wave / C::BLN, wx = wave % C::BLN;
+  int by, bx;
+  block_coords<C>(blockIdx.x, by, bx);
+  const int m0 = by * BM, n0 = bx * BN;
+
+  // One LDS array holds the NST stages.  (No LDS access of this kernel is visible to the compiler as a
+  // load: otherwise it would have to assume that the load may touch a stage a fetch is in flight to
+  // and drain all fetches in front of it.)
+  constexpr int NST = P::NST;
+  __shared__ __attribute__((aligned(1024))) char lds_all[NST * STAGE_BYTES];
+  (void)smem;
+  auto stage_ptr = [&](auto stage_c) -> char* { return lds_all + decltype(stage_c)::value * STAGE_BYTES; };
+
+  // swizzle of a row-contiguous tile (chunk index ^= swz_n(row)).  16-bit: the rows that one pass of a
+  // transposing read touches (k..k+3, and k+8..k+11 with 16-wide matrix-core tiles) must not share banks.
+  // 32-bit: a fragment read is four 32-bit reads; in each, MF lanes read consecutive columns of one row
+  // and the 64/MF lane groups read rows 4 apart, which must fall into different bank ranges.
+  auto swz_n = [](int k, int nch) {
+    if constexpr (ES == 2) return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & (nch - 1);
+    else if constexpr (MF == 32) return (((k >> 2) & 1) << 3) & (nch - 1);
+    else return (((k >> 2) & 3) << 2) & (nch - 1);
+  };
+
+  // ---- fetch: global -> LDS ------------------------------------------------------------------
+  // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
+  // never changes: the K loop spends no vector instruction on addresses.
+  static_assert((long)BM * K * ES < (1L << 31) && (long)BK * M * ES < (1L << 31) && (long)BK * N * ES < (1L << 31),
+                "32-bit lane offsets");
+  unsigned voff_a[NIA], voff_b[NIB];
+#pragma unroll
+  for (int idx = 0; idx < NIA; ++idx) {
+    const int s = 64 * (wave * NIA + idx) + lane;     // physical chunk slot inside the A stage
+    if constexpr (AK) {
+      const int row = s / CHK, cp = s % CHK;
+      const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
+      voff_a[idx] = (unsigned)((row * K + c * G) * ES);
+    } else {
+      const int k = s / NCHA, cp = s % NCHA;
+      const int c = cp ^ swz_n(k, NCHA);
+      voff_a[idx] = (unsigned)((k * M + c * G) * ES);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) {
+    const int s = 64 * (wave * NIB + j) + lane;
+    const int k = s / NCHB, cp = s % NCHB;
+    const int c = cp ^ swz_n(k, NCHB);
+    voff_b[j] = (unsigned)((k * N + c * G) * ES);
+  }
+  const char* const a_base = (const char*)(AK ? A + (long)m0 * K : A + m0);
+  const char* const b_base = (const char*)(B + n0);
+  constexpr long A_KT_BYTES = AK ? (long)BK * ES : (long)BK * M * ES;   // one K tile further
+  constexpr long B_KT_BYTES = (long)BK * N * ES;
+  // The tile bases pass through an empty asm: the compiler must not fold the per-tile scalar part
+  // into the per-lane part (it would hoist "base + lane offset" as a 64-bit vector value and add the
+  // tile offset with vector instructions); kept apart, the fetch uses its scalar-base addressing form.
+  struct TileBase { const char* a; const char* b; };
+  auto tile_base = [&](int kt) {
+    TileBase t = {a_base + kt * A_KT_BYTES, b_base + kt * B_KT_BYTES};
+    asm("" : "+s"(t.a), "+s"(t.b));
+    return t;
+  };
+  auto fetch_item = [&](int idx, const TileBase& tb, auto stage_c) {
+    char* st = stage_ptr(stage_c);
+    if (idx < NIA) {
+      asm volatile("" : "+v"(voff_a[idx]));   // keeps the 32->64 bit extension next to the fetch (see tile_base)
+      const char* src = tb.a + (unsigned long)voff_a[idx];
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + 1024 * (wave * NIA + idx)), 16, 0, 0);
+    } else {
+      const int j = idx - NIA;
+      asm volatile("" : "+v"(voff_b[j]));
+      const char* src = tb.b + (unsigned long)voff_b[j];
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + A_BYTES + 1024 * (wave * NIB + j)), 16, 0, 0);
+    }
+  };
+  constexpr int NFETCH = NIA + NIB;
+
+  // ---- fragments -----------------------------------------------------------------------------
+  // Every fragment read is issued as inline assembly.  As builtins or plain loads the compiler could
+  // not tell that they do not touch the stage a fetch is in flight to and would drain all fetches
+  // (vmcnt(0)) in front of them; it would also insert its own LDS waits, which know nothing of the
+  // reads it cannot see.  The price: the compiler does not know that these reads are asynchronous, so
+  // (1) the K loop counts the reads in flight itself and waits with s_waitcnt lgkmcnt(n) in front of the
+  // matrix-core instructions that consume a fragment, and (2) a fragment stays in the very registers
+  // the read instruction wrote (never a copy made before the data has arrived) until it is consumed.
+  const int frow = lane % MF, fgrp = lane / MF;
+  const int tx = lane % 16;                          // lane inside its 16-lane transposing group
+  const int tsub = (lane / 16) % (MF / 16);          // which 16-column half of the matrix-core tile
+  struct FragTr {                                    // 16-bit, row-contiguous tile: two transposing 64-bit reads
+    u32x2 h[2];
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
+    __device__ __forceinline__ Frag get() const {
+      const u32x4 v = {h[0].x, h[0].y, h[1].x, h[1].y};
+      return __builtin_bit_cast(Frag, v);
+    }
+  };
+  struct FragS4 {                                    // 32-bit, row-contiguous tile: four 32-bit reads
+    unsigned w[4];
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3])); }
+    __device__ __forceinline__ Frag get() const {
+      const u32x4 v = {w[0], w[1], w[2], w[3]};
+      return __builtin_bit_cast(Frag, v);
+    }
+  };
+  struct FragLd {                                    // k-contiguous tile: one 128-bit read
+    u32x4 q;
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(q)); }
+    __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
+  };
+  typedef typename Select<ES == 2, FragTr, FragS4>::type FragRc;
+  typedef typename Select<AK, FragLd, FragRc>::type FragA;
+  typedef FragRc FragB;
+  constexpr int RC_READS = ES == 2 ? 2 : 4;          // LDS instructions per fragment of a row-contiguous tile
+  // LDS address of a fragment read = a per-lane base that never changes (one register per fragment
+  // column block of a row-contiguous tile, one per k-step of a k-contiguous tile) + a compile-time
+  // offset (stage, k-step, fragment row block) that goes into the instruction's 16-bit offset field;
+  // what does not fit the field is added to the base in units of 64 KiB.
+  const unsigned lds0 = (unsigned)(unsigned long)lds_all;
+  // Row-contiguous tile (nch chunks per row at byte offset toff of a stage): a lane reads the G k values
+  // kb .. kb+G-1, kb = s*KS + G*fgrp, of column rowbase + lane%MF.
+  //   16-bit: from two 4(k) x 16(n) blocks, each with one transposing read (16 lanes read a block and
+  //           each receives a column);
+  //   32-bit: one 32-bit read per k value.
+  // The swizzle of a row depends on the lane only (swz_n looks at k bits that s and the read number do
+  // not change).
+  auto rc_lane_base = [&](int toff, int nch, int rowbase) {
+    if constexpr (ES == 2) {
+      const int n = rowbase + 16 * tsub + 4 * (tx % 4);
+      const int k = 8 * fgrp + tx / 4;
+      return lds0 + (unsigned)(toff + (k * nch + ((n / 8) ^ swz_n(k, nch))) * 16 + (n % 8) * 2);
+    } else {
+      const int n = rowbase + frow;
+      const int k = 4 * fgrp;
+      return lds0 + (unsigned)(toff + (k * nch + ((n / 4) ^ swz_n(k, nch))) * 16 + (n % 4) * 4);
+    }
+  };
+  unsigned b_lane[TNI];
+#pragma unroll
+  for (int j = 0; j < TNI; ++j) b_lane[j] = rc_lane_base(A_BYTES, NCHB, wx * WN + j * MF);
+  constexpr int NALANE = AK ? SPW : TMI;
+  unsigned a_lane[NALANE];
+  if constexpr (AK) {
+#pragma unroll
+    for (int st = 0; st < SPW; ++st)
+      a_lane[st] = lds0 + (unsigned)(LK::slot(wy * WM + frow, st * KH + fgrp) * 16);   // swizzle: row%16 = frow%16 only
+  } else {
+#pragma unroll
+    for (int i = 0; i < TMI; ++i) a_lane[i] = rc_lane_base(0, NCHA, wy * WM + i * MF);
+  }
+  auto split_base = [](unsigned lane_base, int imm) { return lane_base + (unsigned)(imm / 65536) * 65536u; };
+  auto read_rc = [&](unsigned lane_base, auto imm_c, auto nch_c, FragRc* dst) {
+    constexpr int IMM0 = decltype(imm_c)::value, ROW = decltype(nch_c)::value * 16;   // bytes per tile row
+    if constexpr (ES == 2) {
+      constexpr int IMM1 = IMM0 + 4 * ROW;                              // second block: four rows further
+      const unsigned base0 = split_base(lane_base, IMM0), base1 = split_base(lane_base, IMM1);
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[0]) : "v"(base0), "n"(IMM0 % 65536));
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst->h[1]) : "v"(base1), "n"(IMM1 % 65536));
+    } else {
+      constexpr int IMM1 = IMM0 + ROW, IMM2 = IMM0 + 2 * ROW, IMM3 = IMM0 + 3 * ROW;   // one tile row per k value
+      const unsigned base0 = split_base(lane_base, IMM0), base1 = split_base(lane_base, IMM1);
+      const unsigned base2 = split_base(lane_base, IMM2), base3 = split_base(lane_base, IMM3);
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[0]) : "v"(base0), "n"(IMM0 % 65536));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[1]) : "v"(base1), "n"(IMM1 % 65536));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[2]) : "v"(base2), "n"(IMM2 % 65536));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst->w[3]) : "v"(base3), "n"(IMM3 % 65536));
+    }
+  };
+  // fragment f of k-step s of the stage: s, f and the stage are compile-time constants (IntC)
+  auto load_a = [&](auto stage_c, auto s_c, auto f_c, FragA* dst) {
+    constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
+    if constexpr (AK) {
+      constexpr int IMM = ST * STAGE_BYTES + F * MF * CHK * 16;
+      const unsigned base = split_base(a_lane[S], IMM);
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst->q) : "v"(base), "n"(IMM % 65536));
+    } else {
+      read_rc(a_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHA * 16>(), IntC<NCHA>(), dst);
+    }
+  };
+  auto load_b = [&](auto stage_c, auto s_c, auto f_c, FragB* dst) {
+    constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
+    read_rc(b_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHB * 16>(), IntC<NCHB>(), dst);
+  };
+  // lgkmcnt(0): every LDS read issued so far has returned
+  auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
+
+  Acc acc[TMI][TNI];
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j)
+#pragma unroll
+      for (int e = 0; e < (int)(sizeof(Acc) / sizeof(float)); ++e) acc[i][j][e] = 0.0f;
+  // The zeros must be in their registers here and now: left alone the compiler writes them right in
+  // front of the first matrix-core instruction of each accumulator, and that instruction (which the
+  // compiler does not recognise as one, see Mfma::run_tied) would need wait states after such a write.
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j) asm volatile("" : "+a"(acc[i][j]));
+  asm volatile("s_nop 7" ::: "memory");
+
+  // ---- K loop ----------------------------------------------------------------------------------
+  // Time line of a k-step: its NM = TMI x TNI matrix-core instructions, row by row (row i: fragment
+  // A_i against B_0..B_TNI-1).  Side work is pinned to slots of that time line:
+  //   * the A fragment that row i+DA needs is read when row i starts (rows >= TMI: rows of the next
+  //     step); it replaces the fragment of a row that is done, so A takes TMI fragments of registers;
+  //   * the B fragments of the next step are read into the other half of a double buffer in the slots
+  //     slot_b(j) of rows RB..TMI-2 (RB = TMI-DA);
+  //   * in the last step of a tile the barrier stands where row RB starts: all reads of this stage
+  //     have been issued by then, and everything read from there on belongs to the next tile;
+  //   * fetches: see below.
+  // LDS reads return in order, so "fragment X has arrived" is "at most n reads issued after X are
+  // still in flight"; n is a compile-time property of this schedule (StreamPlan::allowed).
+#ifndef KCG_SCHED_A_AHEAD
+#define KCG_SCHED_A_AHEAD 0           /* rows an A fragment is read ahead of its use; 0 = TMI-1 */
+#endif
+  // (the further ahead, the earlier the barrier stands in the last step and the more room the fetches
+  // behind it have; measured best at the maximum)
+  constexpr int DA = cmax(1, cmin(TMI - 1, KCG_SCHED_A_AHEAD > 0 ? KCG_SCHED_A_AHEAD : TMI - 1));
+  typedef StreamPlan<TMI, TNI, DA, (AK ? 1 : RC_READS), RC_READS> SP;
+  constexpr int RB = SP::RB;
+  constexpr int MT = SPW * NM;
+  constexpr int BAR = (SPW - 1) * NM + RB * TNI;
+  constexpr int TAIL = MT - BAR;
+  static_assert(TMI >= 2, "the streaming schedule needs two rows of matrix-core tiles per wave");
+  static_assert((NST * SPW) % 2 == 0, "B double buffer: the parity of a step must follow from its stage");
+  // s_waitcnt vmcnt(n), everything else unconstrained: n fetches of this wave may still be in flight
+  static_assert((NST - 2) * NFETCH < 64, "vmcnt has 6 bits");
+  auto vmcnt_only = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
+  auto tiles_ahead = [](int t) {
+    const int last = cmin(KT - 1, t == 0 ? NST - 1 : t - 1 + NST);   // newest tile whose fetch has been issued
+    return cmax(0, last - (t + 1));
+  };
+
+  // prologue: tile 0 -> stage 0, wait for it; then tiles 1..NST-1 in flight
+#pragma unroll
+  for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(0), IntC<0>());
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's chunks of tile 0 are in LDS
+  __syncthreads();
+  static_for<1, NST>([&](auto t) {
+    if (decltype(t)::value < KT) {
+#pragma unroll
+      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t);
+    }
+  });
+  FragA fa[TMI];
+  FragB fb[2][TNI];
+  static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
+  static_for<0, DA>([&](auto i) { load_a(IntC<0>(), IntC<0>(), i, &fa[decltype(i)::value]); });
+  wait_lds();   // the counted waits of the loop assume that nothing older than its own reads is in flight
+
+  // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists; HP: the
+  // fetch of tile kt-1+NST, begun behind the previous tile's barrier, is still being issued.
+  //
+  // A stage is free once the barrier of the tile that computed from it has been passed, and the tile
+  // fetched into it is needed NST-1 barriers later.  With three or more stages its NFETCH fetch
+  // instructions are spread over the whole period up to the next barrier (the memory pipeline of a CU
+  // takes 16 cycles per 1 KiB fetch instruction; four waves issuing all of theirs right behind the
+  // barrier would stall on it); with two stages they must all be issued in the rest of this tile.
+  constexpr int SPREAD = NST >= 3 ? MT : TAIL;
+  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c) {
+    constexpr int CUR = decltype(cur_c)::value;
+    constexpr int NXT = (CUR + 1) % NST, PRV = (CUR + NST - 1) % NST;
+    constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
+    constexpr bool HP = decltype(hasp)::value && SPREAD > TAIL;
+    const TileBase tbn = tile_base(HN ? kt + NST : 0);
+    const TileBase tbp = tile_base(HP ? kt - 1 + NST : 0);
+    static_for<0, SPW>([&](auto s_c) {
+      constexpr int S = decltype(s_c)::value;
+      constexpr bool LAST = (S == SPW - 1);
+      constexpr int PB = (CUR * SPW + S) & 1;       // half of the B double buffer this step computes from
+      constexpr bool NEXT = !LAST || H1;            // a next step exists, its fragments are read under this one
+      static_for<0, TMI>([&](auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        // the fragments of this row have arrived.  Without a next step the reads the count relies on
+        // are not issued: wait for everything instead.
+        if constexpr (NEXT) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(SP::allowed(I)) : "memory");
+        else wait_lds();
+        if constexpr (LAST && I == RB) {
+          // tile kt+1 has landed (this wave's part): of the fetches issued so far only those of the
+          // tiles behind it may still be in flight
+          if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
+          wait_lds();        // this wave's reads of stage CUR have all returned
+          // ... everyone's part; and every wave is done reading stage CUR.  The bare barrier instruction:
+          // __syncthreads() comes with a fence in front of which the compiler drains every fetch in
+          // flight (vmcnt(0)), which would expose the whole memory latency at each tile.  What has
+          // to be complete at this point is exactly what the two waits above ask for.
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+        }
+        // the empty asm statements make the fragments "outputs" of the wait: the matrix-core
+        // instructions that consume them cannot be scheduled in front of it
+        fa[I].pin();
+        if constexpr (I == 0) {
+#pragma unroll
+          for (int j = 0; j < TNI; ++j) fb[PB][j].pin();
+        }
+        if constexpr (I + DA < TMI) load_a(IntC<CUR>(), IntC<S>(), IntC<I + DA>(), &fa[I + DA]);
+        else if constexpr (!LAST) load_a(IntC<CUR>(), IntC<S + 1>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
+        else if constexpr (H1) load_a(IntC<NXT>(), IntC<0>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
+        static_for<0, TNI>([&](auto j_c) {
+          constexpr int J = decltype(j_c)::value;
+          constexpr int slot = S * NM + I * TNI + J;
+          // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
+          // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
+          // odd rows run right to left: neighbours on the time line always share one operand
+          constexpr int JC = (I & 1) ? TNI - 1 - J : J;
+          MI::run_tied(acc[I][JC], fb[PB][JC].get(), fa[I].get());
+          static_for<0, TNI>([&](auto jj_c) {
+            constexpr int JJ = decltype(jj_c)::value;
+            if constexpr (SP::slot_b(JJ) == I * TNI + J) {
+              if constexpr (!LAST) load_b(IntC<CUR>(), IntC<S + 1>(), jj_c, &fb[PB ^ 1][JJ]);
+              else if constexpr (H1) load_b(IntC<NXT>(), IntC<0>(), jj_c, &fb[PB ^ 1][JJ]);
+            }
+          });
+#pragma unroll
+          for (int f = 0; f < NFETCH; ++f) {
+            const int pos = BAR + (f * SPREAD) / NFETCH;          // position on the time line that starts at this tile
+            if (HN && pos == slot) fetch_item(f, tbn, IntC<CUR>());
+            if (HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>());
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      });
+    });
+  };
+  // Tile 0 first (nothing of an earlier period to continue); then groups of NST tiles that have every
+  // neighbour; the rest is unrolled with the right flags at compile time (KT is a constant).
+  // tiles_ahead(T): how many tiles behind tile T+1 have been issued when tile T reaches its barrier
+  // (the prologue issued tiles 0..NST-1, tile t issues or completes the issue of tile t-1+NST)
+  tile(0, IntC<0>(), BoolC<(1 < KT)>(), BoolC<(NST < KT)>(), BoolC<false>(), IntC<tiles_ahead(0)>());
+  constexpr int NFULL = KT - NST - 1 > 0 ? KT - NST - 1 : 0;   // tiles 1 .. KT-NST-1 have kt+NST < KT
+  constexpr int NG = NFULL / NST;
+  for (int g = 0; g < NG; ++g) {
+    static_for<0, NST>([&](auto sc) {
+      constexpr int S = decltype(sc)::value;
+      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>());
+    });
+  }
+  static_for<1 + NG * NST, KT>([&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+    tile(T, IntC<T % NST>(), BoolC<(T + 1 < KT)>(), BoolC<(T + NST < KT)>(), BoolC<(T - 1 + NST < KT)>(), IntC<tiles_ahead(T)>());
+  });
+
+  // the last matrix-core results must have left the pipeline before the epilogue reads them (the
+  // compiler, which normally inserts these wait states, does not know the instructions above)
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  // ---- epilogue --------------------------------------------------------------------------------
+  // With swapped operands a 32x32 accumulator holds, per lane, row m = lane%32 and columns
+  // n = 8*g + 4*(lane/32) + {0..3} for g = 0..3 (16x16: row lane%16, columns 4*(lane/16) + {0..3}).
+  constexpr int NACC = (int)(sizeof(Acc) / sizeof(float));
+  const int orow = lane % MF;
+  const int ocol = (lane / MF) * 4;
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j)
+#pragma unroll
+      for (int g = 0; g < NACC / 4; ++g) {
+        const int row = m0 + wy * WM + i * MF + orow;
+        const int col = n0 + wx * WN + j * MF + g * 8 + ocol;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
+        gstore<TC, float, 4, false, true>(Cm, v, row, col, N, M, N);
+      }
+}
+
+}  // namespace kcg
