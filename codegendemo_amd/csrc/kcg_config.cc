@@ -236,6 +236,8 @@ bool mfma_direct(const MatmulConfig& c) {
   if (!is_pow2(c.BM) || !is_pow2(c.BN) || !is_pow2(c.BK) || c.BM < 64 || c.BN < 64) return false;
   if ((c.BM * c.BK / g) % (64 * nw) || (c.BN * c.BK / g) % (64 * nw)) return false;
   if (c.M % g || c.N % g || c.K % g) return false;
+  const long lim = 1L << 31;                              // 32-bit byte offsets per lane inside a tile panel
+  if ((long)c.BM * c.K * es >= lim || (long)c.BK * c.M * es >= lim || (long)c.BK * c.N * es >= lim) return false;
   return 2 * (c.BM + c.BN) * c.BK * es <= kMaxLdsBytes;
 }
 

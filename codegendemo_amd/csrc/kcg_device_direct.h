@@ -7,21 +7,21 @@
 namespace kcg {
 
 // =============================================================================================
-// Family 2b: matrix-core kernel with direct global->LDS staging (16-bit inputs).
+// Family 2b: matrix-core kernel with direct global->LDS staging.
 //
-// Every lane fetches one 16-byte chunk with global_load_lds_dwordx4; a wave's 64 chunks land in 1 KiB of
-// consecutive LDS, so no register, no ds_write and no VALU work is spent on staging and the fetch of
-// tile kt+2 can be in flight for a whole K tile.  The LDS image keeps the orientation of global memory:
-//   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/8 chunks of 8 k values each; a fragment
+// Every lane fetches one 16-byte chunk (G = 4 fp32 or 8 fp16/bf16 elements) with
+// global_load_lds_dwordx4; a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
+// ds_write and no vector ALU work is spent on staging, and with NST stages the fetch of a tile can be in
+// flight for NST-1 K tiles.  The LDS image keeps the orientation of global memory:
+//   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/G chunks of G k values each; a fragment
 //                                           is one ds_read_b128 (as in gemm_mfma)
-//   row-contiguous operand (B; A^T)       : rows = k, NCH = BN/8 (BM/8) chunks of 8 n values each; a
-//                                           fragment is two ds_read_b64_tr_b16: 16 lanes read a 4(k) x
-//                                           16(n) block and each lane receives one column of it, which
-//                                           is the k-packed layout the matrix core wants
+//   row-contiguous operand (B; A^T)       : rows = k, NCH = BN/G (BM/G) chunks of G n values each.
+//       16-bit: a fragment is two ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n) block and each lane
+//               receives one column of it, which is the k-packed layout the matrix core wants
+//       32-bit: a fragment is four ds_read_b32, one per k value
 // The bank swizzle is applied on the fetch side: the lane that fills physical chunk c' of a row fetches
 // logical chunk c' ^ swz(row), and readers look chunk c up at c ^ swz(row).
 // =============================================================================================
-typedef short short4v __attribute__((ext_vector_type(4)));
 
 // Static schedule of the fragment reads of one k-step of the direct-staging kernel (see its K loop):
 // which slot reads which B fragment of the next step, and how many LDS read instructions issued after
@@ -83,7 +83,9 @@ struct DirectPlan {
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
       SPW > 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
       (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
-      (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024;
+      (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
+      // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
+      (long)C::BM * C::K * ES < (1L << 31) && (long)C::BK * C::M * ES < (1L << 31) && (long)C::BK * C::N * ES < (1L << 31);
   // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles); an even number
   // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
   static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * ES;
@@ -154,8 +156,6 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
   // never changes: the K loop spends no vector instruction on addresses.
-  static_assert((long)BM * K * ES < (1L << 31) && (long)BK * M * ES < (1L << 31) && (long)BK * N * ES < (1L << 31),
-                "32-bit lane offsets");
   unsigned voff_a[NIA], voff_b[NIB];
 #pragma unroll
   for (int idx = 0; idx < NIA; ++idx) {
