@@ -241,6 +241,18 @@ def main():
                                     "frac": ach16 / PEAK_TFLOPS["f16"], "traffic": measured_traffic(info16["kernel_name"]),
                                     "launch_ms": ms_launch16}}
 
+        # the same config with bfloat16 inputs (same kernel template, same data distribution)
+        cfgb = dict(cfg16)
+        cfgb["DATATYPE_A"] = cfgb["DATATYPE_B"] = 3
+        kpmb, kernelb, infob = build_kernel(cfgb)
+        _, _, Ab, Bb, Cb = make_inputs(kpmb, "normal")
+        ms_stepb, ms_launchb = time_steps(kernelb, Ab, Bb, Cb, args.steps, args.warmup)
+        achb = flops / (ms_launchb * 1e-3) / 1e12
+        out["bf16"] = {"value": flops / (ms_stepb * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_stepb,
+                       "dtype": "bf16 in, f32 accumulate/out", "kernel": infob["kernel_name"],
+                       "roofline": {"bound": "mfma", "achieved": achb, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                                    "frac": achb / PEAK_TFLOPS["f16"], "launch_ms": ms_launchb}}
+        del Ab, Bb, Cb
         # What the matrix pipeline alone sustains on this box (register operands, no memory traffic), on
         # zeros and on data like the workload's: the stand-alone runner measures it in a child process.
         # fp16 GEMMs on this part run at its power limit, so the second figure bounds any fp16 kernel.
