@@ -82,6 +82,10 @@ EXACT_CASES = [
                                       shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-mf16-8w-at1", MFMA, dict(M=256, N=256, K=544, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=1,
                                           shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-kt1", MFMA, dict(M=256, N=256, K=16, BM=128, BN=128, TM=8, TN=8, BK=16, is_atrans=0,
+                                  shared_prefetch=1, reg_prefetch=1)),                    # a single K tile
+    ("f32-direct-kt2-at1", MFMA, dict(M=256, N=256, K=64, BM=128, BN=128, TM=8, TN=8, BK=32, is_atrans=1,
+                                      shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-1wave", MFMA, dict(M=256, N=256, K=1056, BM=128, BN=128, TM=16, TN=16, BK=32, is_atrans=0,
                                     shared_prefetch=1, reg_prefetch=1)),
     # fp64 on the matrix cores (16x16x4 instructions, two k values per 16-byte chunk)
@@ -148,6 +152,10 @@ HALF_CASES = [
                               BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-2rows-at1", dict(M=192, N=128, K=736, dtype=2, dtype_c=4, is_atrans=1, BM=64, BN=64, TM=4, TN=4,
                                   BK=32, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-kt1", dict(M=256, N=256, K=64, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
+                            shared_prefetch=1, reg_prefetch=1)),                          # a single K tile
+    ("bf16-direct-kt3-at1", dict(M=256, N=256, K=96, dtype=3, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8, BK=32,
+                                 shared_prefetch=1, reg_prefetch=1)),
     # one wave per block: 32 fetch instructions per wave and tile limit the number of stages in flight
     ("f16-direct-1wave", dict(M=256, N=256, K=1088, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=16, TN=16,
                               BK=64, shared_prefetch=1, reg_prefetch=1)),
