@@ -1,0 +1,1 @@
+"""Operator descriptions of the kcg mirror (matmul)."""

@@ -1,0 +1,1 @@
+"""Test suite: CPU tests (oracle, config semantics, ABI, tuner loop) and GPU parity tests (marker gpu)."""
