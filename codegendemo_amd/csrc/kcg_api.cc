@@ -412,16 +412,16 @@ static long code_object_scratch_bytes(const std::vector<char>& code) {
   return -1;
 }
 
-int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, kcg_kernel_info* out) {
-  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
-  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
-  std::string why;
-  int k = resolve_kind(c, kind, &why);
-  if (k < 0) return fail(k, "invalid config: " + why);
-  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
+// Outcome of build_variant besides the kcg_status values: the direct-staging build would spill.
+static const int kBuildSpills = 1;
+
+// Builds (or finds in the cache) the code object of config c as kernel family k; `allow_direct` lets a
+// matrix-core config that is eligible for direct global->LDS staging use that kernel.
+static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, const std::string& arch, kcg_kernel_info* out) {
   const bool xcd = env_flag("KCG_XCD_REMAP", true);
+  const bool direct = allow_direct && k == KCG_KIND_MFMA && kcg::mfma_direct(c);
   const std::string name = kcg::kernel_name(c);
-  const std::string stub = kcg::instantiation_source(c, k, xcd);
+  const std::string stub = kcg::instantiation_source(c, k, xcd, allow_direct);
 
   memset(out, 0, sizeof(*out));
   if (name.size() >= sizeof(out->kernel_name)) return fail(KCG_ERR_ARGUMENT, "kernel name too long");
@@ -430,7 +430,7 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   out->grid[1] = out->grid[2] = 1;
   out->block[0] = c.thread_num();
   out->block[1] = out->block[2] = 1;
-  out->lds_bytes = kcg::lds_bytes(c, k);
+  out->lds_bytes = kcg::lds_bytes(c, k, allow_direct);
   out->kind = k;
 
   if (!rtc_api().ok) return fail(KCG_ERR_COMPILE, "hiprtc unavailable:" + rtc_api().error);
@@ -455,11 +455,16 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   const std::string path = dir + "/" + name + "." + hex + ".hsaco";
   if (path.size() >= sizeof(out->code_path)) return fail(KCG_ERR_IO, "code object path too long");
   memcpy(out->code_path, path.c_str(), path.size() + 1);
+  // remembers that this very build (same sources, flags, compiler) spilled: no need to compile it again
+  const std::string spill_marker = dir + "/" + name + "." + hex + ".spills";
 
-  if (file_exists(path) && !env_flag("KCG_CACHE_BYPASS", false)) {
-    out->cache_hit = 1;
-    g_err.clear();
-    return KCG_OK;
+  if (!env_flag("KCG_CACHE_BYPASS", false)) {
+    if (file_exists(path)) {
+      out->cache_hit = 1;
+      g_err.clear();
+      return KCG_OK;
+    }
+    if (direct && file_exists(spill_marker)) return kBuildSpills;
   }
 
   hiprtcProgram prog;
@@ -489,12 +494,11 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   if (r != HIPRTC_SUCCESS || n == 0) return fail(KCG_ERR_COMPILE, "hiprtc returned no code object");
   // The direct-staging kernel reads LDS with instructions the compiler does not know to be
   // asynchronous: a fragment register spilled to scratch memory would be stored before its data has
-  // arrived.  Such a build is refused (and not cached) instead of returning wrong products.
-  if (k == KCG_KIND_MFMA && kcg::mfma_direct(c)) {
-    const long scratch = code_object_scratch_bytes(code);
-    if (scratch > 0)
-      return fail(KCG_ERR_COMPILE, "direct-staging kernel " + name + " needs " + std::to_string(scratch) +
-                                       " bytes of scratch memory per lane (register spills); use a smaller tile");
+  // arrived.  Such a build is never used (nor cached): the caller falls back to register staging.
+  if (direct && code_object_scratch_bytes(code) > 0) {
+    const char note[] = "direct-staging build needs scratch memory (register spills); register staging is used instead\n";
+    write_file_atomic(spill_marker, note, sizeof(note) - 1);
+    return kBuildSpills;
   }
   if (!write_file_atomic(path, code.data(), code.size())) return fail(KCG_ERR_IO, "cannot write " + path);
   if (env_flag("KCG_KEEP_SOURCE", false)) {
@@ -504,6 +508,19 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   g_err.clear();
   return KCG_OK;
 }
+
+int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, kcg_kernel_info* out) {
+  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  std::string why;
+  int k = resolve_kind(c, kind, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
+  int r = build_variant(c, k, /*allow_direct=*/true, arch, out);
+  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, out);
+  return r;
+}
+
 
 int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int device, uint64_t* module,
              uint64_t* function, int32_t* n_regs, int32_t* n_spills) {

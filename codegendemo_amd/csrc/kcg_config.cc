@@ -241,8 +241,8 @@ bool mfma_direct(const MatmulConfig& c) {
   return 2 * (c.BM + c.BN) * c.BK * es <= kMaxLdsBytes;
 }
 
-int lds_bytes(const MatmulConfig& c, int kind) {
-  if (kind == KCG_KIND_MFMA && mfma_direct(c)) return 0;   // that path declares its stages statically
+int lds_bytes(const MatmulConfig& c, int kind, bool allow_direct) {
+  if (allow_direct && kind == KCG_KIND_MFMA && mfma_direct(c)) return 0;   // that path declares its stages statically
   const int stages = c.SHMP ? 2 : 1;
   const int szA = dtype_size(c.dtA), szB = dtype_size(c.dtB);
   const int accsz = (c.dtC == KCG_DT_FLOAT64) ? 8 : 4;
@@ -275,7 +275,7 @@ void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int*
   }
 }
 
-std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap) {
+std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap, bool allow_direct) {
   std::ostringstream s;
   const char* acc = (c.dtC == KCG_DT_FLOAT64) ? "double" : "float";
   s << "// generated by libkcg_gemm: instantiation of the " << (kind == KCG_KIND_MFMA ? "gemm_mfma" : "gemm_simt")
@@ -299,7 +299,8 @@ std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap
   Bv("ATRANS", c.ATRANS != 0);
   Bv("EDGE", c.edge());
   Bv("XCD_REMAP", xcd_remap);
-  Bv("DIRECT", kind == KCG_KIND_MFMA && mfma_direct(c));
+  Bv("DIRECT_ELIGIBLE", kind == KCG_KIND_MFMA && mfma_direct(c));   // the rule; the device header re-derives and compares it
+  Bv("DIRECT", allow_direct && kind == KCG_KIND_MFMA && mfma_direct(c));
   I("SIMT_PAD_A", simt_pad_a(c)); I("SIMT_PAD_B", 0);
   s << "};\n}  // namespace\n\n";
   s << "extern \"C\" __global__ __launch_bounds__(" << c.thread_num() << ") void " << kernel_name(c)

@@ -54,11 +54,11 @@ std::string kernel_name(const MatmulConfig& c);
 int reference_lds_bytes(const MatmulConfig& c);
 int simt_pad_a(const MatmulConfig& c);
 bool mfma_direct(const MatmulConfig& c);      // matrix-core kernel stages operands with direct global->LDS loads
-int lds_bytes(const MatmulConfig& c, int kind);  // what the chosen kernel family really needs
+int lds_bytes(const MatmulConfig& c, int kind, bool allow_direct = true);  // what the chosen kernel really needs
 void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int* bx);
 
 // HIP text of the instantiation stub for (config, kind, xcd_remap).
-std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap);
+std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap, bool allow_direct = true);
 
 constexpr int kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KiB LDS per CU, one workgroup may take all
 constexpr int kMaxThreads = 1024;

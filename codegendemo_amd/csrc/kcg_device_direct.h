@@ -97,8 +97,10 @@ struct DirectPlan {
   static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
   static constexpr int NST_CAP = NST_MAX < 2 ? 2 : (NST_MAX > 4 ? 4 : NST_MAX);
   static constexpr int NST = (SPW % 2 == 1 && NST_CAP % 2 == 1) ? NST_CAP - 1 : NST_CAP;
-  // the host picks the path (it must size dynamic LDS accordingly); both sides have to agree
-  static_assert(ELIGIBLE == C::DIRECT, "host and device disagree on the direct-staging eligibility rule");
+  // the host picks the path (it must size dynamic LDS accordingly): both sides have to agree on the
+  // rule; the host may still decline an eligible config (a direct-staging build that would spill)
+  static_assert(ELIGIBLE == C::DIRECT_ELIGIBLE, "host and device disagree on the direct-staging eligibility rule");
+  static_assert(ELIGIBLE || !C::DIRECT, "direct staging asked for an ineligible config");
   static constexpr bool OK = C::DIRECT;
 };
 

@@ -126,8 +126,10 @@ int kcg_block_mapping(const kcg_matmul_cfg* cfg, int bid, int xcd_remap, int32_t
  * kind, arch and kernel source is a cache hit and does not compile.  `kind` is a kcg_kernel_kind.
  * Thread-safe and re-entrant; needs no GPU.
  * KCG_ERR_INVALID_CONFIG: the config breaks a rule (text says which), nothing was compiled.
- * KCG_ERR_COMPILE: hiprtc failed, or the config selects the direct-staging kernel and its build would
- * spill registers to scratch memory (that kernel cannot tolerate spills; no code object is written). */
+ * KCG_ERR_COMPILE: hiprtc failed.
+ * A config that selects the direct-staging kernel but whose build would spill registers to scratch memory
+ * (that kernel cannot tolerate spills) silently gets the register-staged kernel instead; a
+ * "<name>.<hash>.spills" marker in the cache directory remembers the decision. */
 int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch, int kind, kcg_kernel_info* out);
 
 /* The HIP source text that kcg_compile_matmul would hand to hiprtc for this config (the generated

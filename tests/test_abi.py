@@ -92,15 +92,20 @@ def test_last_error_is_per_thread():
     assert seen["msg"] == ""
 
 
-def test_direct_staging_kernel_that_spills_is_refused(tmp_path, monkeypatch):
+def test_direct_staging_build_that_spills_falls_back_to_register_staging(tmp_path, monkeypatch):
     """The direct-staging kernel reads LDS asynchronously behind the compiler's back; a build whose
-    fragments would be spilled to scratch memory must fail as a compile error and leave no code object."""
+    fragments would be spilled to scratch memory must never be used.  The library notices it in the code
+    object's metadata, remembers it with a marker file and builds the register-staged kernel instead."""
     from codegendemo_amd.kcg.ConfigGenerator import make_config
     from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
     monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path))
     # 8 waves of 128x128 accumulators: 256 registers per lane cannot hold accumulators and fragments
     cfg = make_config(4096, 4096, 4096, dtype=2, dtype_c=4, BM=256, BN=512, BK=32, TM=16, TN=16, is_atrans=0,
                       shared_prefetch=1, reg_prefetch=1)
-    with pytest.raises(_native.KcgError, match="scratch memory"):
-        _native.compile_matmul(kernelArgFromConfig(cfg).values(), "gfx950", _native.KIND_MFMA)
-    assert not [f for f in os.listdir(tmp_path) if f.endswith(".hsaco")]
+    values = kernelArgFromConfig(cfg).values()
+    info = _native.compile_matmul(values, "gfx950", _native.KIND_MFMA)
+    assert info["lds_bytes"] == 2 * (256 + 512) * 32 * 2 and not info["cache_hit"]     # dynamic LDS of the register-staged kernel
+    assert sorted(f.rsplit(".", 1)[1] for f in os.listdir(tmp_path)) == ["hsaco", "spills"]
+    assert "static constexpr bool DIRECT = false;" not in _native.instantiation_source(values, _native.KIND_MFMA)
+    again = _native.compile_matmul(values, "gfx950", _native.KIND_MFMA)                 # marker + cache: nothing is compiled
+    assert again["cache_hit"] and again["code_path"] == info["code_path"]

@@ -66,12 +66,7 @@ def test_random_config_sample_is_bit_exact(oracle):
         a = SI.small_ints((M, K), SI.STREAM_A, lim=2)
         b = SI.small_ints((K, N), SI.STREAM_B, lim=2)
         print(f"[case] random {i} kind={kind} {kernelArgFromConfig(cfg).values()}", flush=True)
-        try:
-            got, info = run_gemm(cfg, a, b, kind)
-        except _native.KcgError as e:
-            if "scratch memory" in str(e):      # a valid config whose direct-staging build would spill: refused by design
-                continue
-            raise
+        got, info = run_gemm(cfg, a, b, kind)
         direct += int(kind == _native.KIND_MFMA and info["lds_bytes"] == 0)
         want = oracle.matmul(a, b, a_trans=False)
         bad = int((got != want).sum()) + int(np.isnan(got).sum())
