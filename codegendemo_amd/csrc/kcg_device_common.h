@@ -125,7 +125,8 @@ struct BlockMap {
 
 // Load VEC consecutive elements T from row r, column c of a row-major matrix with leading dimension
 // LD into dst[0..VEC).  With EDGE, elements outside [0,RMAX) x [0,CMAX) read as zero.  ALIGNED says
-// every such vector is naturally aligned to VEC*sizeof(T) so one wide load is legal.
+// every such vector is naturally aligned to VEC*sizeof(T) so one wide load is legal: LD (which is CMAX
+// at every call site, the matrices being dense) and c are multiples of VEC.
 template <class T, int VEC, bool EDGE, bool ALIGNED>
 __device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r, int c, int LD, int RMAX, int CMAX) {
   if constexpr (!EDGE) {
@@ -135,14 +136,19 @@ __device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r,
 #pragma unroll
       for (int e = 0; e < VEC; ++e) dst[e] = base[(long)r * LD + c + e];
     }
-  } else {
-    if (ALIGNED && r < RMAX && c + VEC <= CMAX) {
+  } else if constexpr (ALIGNED) {
+    // c and CMAX are multiples of VEC: the vector lies inside or outside as a whole (one predicate per
+    // vector instead of one per element)
+    if (r < RMAX && c < CMAX) {
       copy_bytes<VEC * (int)sizeof(T)>(dst, base + (long)r * LD + c);
     } else {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        dst[e] = (r < RMAX && c + e < CMAX) ? base[(long)r * LD + c + e] : T(0);
-      }
+      for (int e = 0; e < VEC; ++e) dst[e] = T(0);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      dst[e] = (r < RMAX && c + e < CMAX) ? base[(long)r * LD + c + e] : T(0);
     }
   }
 }
@@ -160,14 +166,12 @@ __device__ __forceinline__ void gstore(TC* __restrict__ base, const ACC* src, in
 #pragma unroll
       for (int e = 0; e < VEC; ++e) base[(long)r * LD + c + e] = tmp[e];
     }
+  } else if constexpr (ALIGNED) {
+    if (r < RMAX && c < CMAX) copy_bytes<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
   } else {
-    if (ALIGNED && r < RMAX && c + VEC <= CMAX) {
-      copy_bytes<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
-    } else {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e)
-        if (r < RMAX && c + e < CMAX) base[(long)r * LD + c + e] = tmp[e];
-    }
+    for (int e = 0; e < VEC; ++e)
+      if (r < RMAX && c + e < CMAX) base[(long)r * LD + c + e] = tmp[e];
   }
 }
 

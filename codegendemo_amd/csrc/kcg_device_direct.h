@@ -19,6 +19,10 @@ namespace kcg {
 //       16-bit: a fragment is two ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n) block and each lane
 //               receives one column of it, which is the k-packed layout the matrix core wants
 //       32-bit: a fragment is four ds_read_b32, one per k value
+// Edge tiles cost the K loop nothing: a lane whose chunk lies outside the matrix (rows or columns
+// beyond M or N; k beyond K in the last, partial K tile) fetches a chunk of the same tile that does exist
+// instead.  What lands in LDS for it only ever reaches accumulators of rows/columns that are not stored
+// (M, N) or is not read at all (the partial K tile computes only the k-steps it has).
 // The bank swizzle is applied on the fetch side: the lane that fills physical chunk c' of a row fetches
 // logical chunk c' ^ swz(row), and readers look chunk c up at c ^ swz(row).
 // =============================================================================================
@@ -79,9 +83,10 @@ struct DirectPlan {
   static constexpr int SPW = (C::BK % KS == 0) ? C::BK / KS : 0;
   static constexpr bool pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
   static constexpr bool ELIGIBLE =
-      (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && !C::EDGE && C::SHMP && C::REGP && C::LC != 0 &&
+      (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
-      SPW > 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
+      // edge tiles in M and N are fine; K needs one full tile and a remainder of whole k-steps
+      SPW > 0 && C::K >= C::BK && (C::K % C::BK) % KS == 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
       (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
       (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
@@ -115,7 +120,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int WM = P::WM, WN = P::WN, MF = P::MF;
   constexpr int KH = 64 / MF, KS = P::KS, SPW = P::SPW;
   constexpr int TMI = WM / MF, TNI = WN / MF, NM = P::NM, NW = P::NW;
-  constexpr int KT = K / BK;
+  constexpr int KT = K / BK;                            // full K tiles
+  constexpr int KR = K % BK, SPWT = KR / KS;            // the remainder: one more tile of SPWT k-steps
+  constexpr int KTT = KT + (KR > 0 ? 1 : 0);
+  constexpr bool EDGE_M = M % BM != 0, EDGE_N = N % BN != 0;
   constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
   constexpr int ES = P::ES, G = P::G;                   // element size; elements per 16-byte chunk
   constexpr int CHK = BK / G;                           // chunks per row of a k-contiguous tile
@@ -158,27 +166,39 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
   // never changes: the K loop spends no vector instruction on addresses.
-  unsigned voff_a[NIA], voff_b[NIB];
-#pragma unroll
-  for (int idx = 0; idx < NIA; ++idx) {
+  // kvalid: how many k rows/values of the tile exist (BK, or KR for the partial tile)
+  auto off_a = [&](int idx, int kvalid) -> unsigned {
     const int s = 64 * (wave * NIA + idx) + lane;     // physical chunk slot inside the A stage
     if constexpr (AK) {
-      const int row = s / CHK, cp = s % CHK;
-      const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
-      voff_a[idx] = (unsigned)((row * K + c * G) * ES);
+      int row = s / CHK;
+      const int cp = s % CHK;
+      int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
+      if (c * G >= kvalid) c = 0;
+      if constexpr (EDGE_M) row = cmin(row, M - 1 - m0);
+      return (unsigned)((row * K + c * G) * ES);
     } else {
-      const int k = s / NCHA, cp = s % NCHA;
-      const int c = cp ^ swz_n(k, NCHA);
-      voff_a[idx] = (unsigned)((k * M + c * G) * ES);
+      int k = s / NCHA;
+      const int cp = s % NCHA;
+      int c = cp ^ swz_n(k, NCHA);
+      if (k >= kvalid) k = 0;
+      if constexpr (EDGE_M) c = cmin(c, (M - m0) / G - 1);
+      return (unsigned)((k * M + c * G) * ES);
     }
-  }
-#pragma unroll
-  for (int j = 0; j < NIB; ++j) {
+  };
+  auto off_b = [&](int j, int kvalid) -> unsigned {
     const int s = 64 * (wave * NIB + j) + lane;
-    const int k = s / NCHB, cp = s % NCHB;
-    const int c = cp ^ swz_n(k, NCHB);
-    voff_b[j] = (unsigned)((k * N + c * G) * ES);
-  }
+    int k = s / NCHB;
+    const int cp = s % NCHB;
+    int c = cp ^ swz_n(k, NCHB);
+    if (k >= kvalid) k = 0;
+    if constexpr (EDGE_N) c = cmin(c, (N - n0) / G - 1);
+    return (unsigned)((k * N + c * G) * ES);
+  };
+  unsigned voff_a[NIA], voff_b[NIB];
+#pragma unroll
+  for (int idx = 0; idx < NIA; ++idx) voff_a[idx] = off_a(idx, BK);
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) voff_b[j] = off_b(j, BK);
   const char* const a_base = (const char*)(AK ? A + (long)m0 * K : A + m0);
   const char* const b_base = (const char*)(B + n0);
   constexpr long A_KT_BYTES = AK ? (long)BK * ES : (long)BK * M * ES;   // one K tile further
@@ -192,17 +212,29 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     asm("" : "+s"(t.a), "+s"(t.b));
     return t;
   };
-  auto fetch_item = [&](int idx, const TileBase& tb, auto stage_c) {
+  // partial_c: the tile fetched is the partial one behind the last full K tile
+  auto fetch_item = [&](int idx, const TileBase& tb, auto stage_c, auto partial_c) {
+    constexpr bool PARTIAL = decltype(partial_c)::value;
     char* st = stage_ptr(stage_c);
     if (idx < NIA) {
-      asm volatile("" : "+v"(voff_a[idx]));   // keeps the 32->64 bit extension next to the fetch (see tile_base)
-      const char* src = tb.a + (unsigned long)voff_a[idx];
+      unsigned off;
+      if constexpr (PARTIAL) off = off_a(idx, KR);
+      else {
+        asm volatile("" : "+v"(voff_a[idx]));   // keeps the 32->64 bit extension next to the fetch (see tile_base)
+        off = voff_a[idx];
+      }
+      const char* src = tb.a + (unsigned long)off;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(st + 1024 * (wave * NIA + idx)), 16, 0, 0);
     } else {
       const int j = idx - NIA;
-      asm volatile("" : "+v"(voff_b[j]));
-      const char* src = tb.b + (unsigned long)voff_b[j];
+      unsigned off;
+      if constexpr (PARTIAL) off = off_b(j, KR);
+      else {
+        asm volatile("" : "+v"(voff_b[j]));
+        off = voff_b[j];
+      }
+      const char* src = tb.b + (unsigned long)off;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(st + A_BYTES + 1024 * (wave * NIB + j)), 16, 0, 0);
     }
@@ -362,19 +394,19 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   static_assert((NST - 2) * NFETCH < 64, "vmcnt has 6 bits");
   auto vmcnt_only = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
   auto tiles_ahead = [](int t) {
-    const int last = cmin(KT - 1, t == 0 ? NST - 1 : t - 1 + NST);   // newest tile whose fetch has been issued
+    const int last = cmin(KTT - 1, t == 0 ? NST - 1 : t - 1 + NST);  // newest tile whose fetch has been issued
     return cmax(0, last - (t + 1));
   };
 
   // prologue: tile 0 -> stage 0, wait for it; then tiles 1..NST-1 in flight
 #pragma unroll
-  for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(0), IntC<0>());
+  for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(0), IntC<0>(), BoolC<false>());
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's chunks of tile 0 are in LDS
   __syncthreads();
   static_for<1, NST>([&](auto t) {
-    if (decltype(t)::value < KT) {
+    if (decltype(t)::value < KTT) {
 #pragma unroll
-      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t);
+      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t, BoolC<(KR > 0 && decltype(t)::value == KT)>());
     }
   });
   FragA fa[TMI];
@@ -384,7 +416,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   wait_lds();   // the counted waits of the loop assume that nothing older than its own reads is in flight
 
   // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists; HP: the
-  // fetch of tile kt-1+NST, begun behind the previous tile's barrier, is still being issued.
+  // fetch of tile kt-1+NST, begun behind the previous tile's barrier, is still being issued.  NS: k-steps
+  // of this tile (SPW, fewer for the partial tile); PN / PP: the tile fetched under HN / HP is the partial one.
   //
   // A stage is free once the barrier of the tile that computed from it has been passed, and the tile
   // fetched into it is needed NST-1 barriers later.  With three or more stages its NFETCH fetch
@@ -392,16 +425,16 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // takes 16 cycles per 1 KiB fetch instruction; four waves issuing all of theirs right behind the
   // barrier would stall on it); with two stages they must all be issued in the rest of this tile.
   constexpr int SPREAD = NST >= 3 ? MT : TAIL;
-  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c) {
-    constexpr int CUR = decltype(cur_c)::value;
+  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c, auto ns_c, auto pn_c, auto pp_c) {
+    constexpr int CUR = decltype(cur_c)::value, NS = decltype(ns_c)::value;
     constexpr int NXT = (CUR + 1) % NST, PRV = (CUR + NST - 1) % NST;
     constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
     constexpr bool HP = decltype(hasp)::value && SPREAD > TAIL;
     const TileBase tbn = tile_base(HN ? kt + NST : 0);
     const TileBase tbp = tile_base(HP ? kt - 1 + NST : 0);
-    static_for<0, SPW>([&](auto s_c) {
+    static_for<0, NS>([&](auto s_c) {
       constexpr int S = decltype(s_c)::value;
-      constexpr bool LAST = (S == SPW - 1);
+      constexpr bool LAST = (S == NS - 1);
       constexpr int PB = (CUR * SPW + S) & 1;       // half of the B double buffer this step computes from
       constexpr bool NEXT = !LAST || H1;            // a next step exists, its fragments are read under this one
       static_for<0, TMI>([&](auto i_c) {
@@ -451,8 +484,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 #pragma unroll
           for (int f = 0; f < NFETCH; ++f) {
             const int pos = BAR + (f * SPREAD) / NFETCH;          // position on the time line that starts at this tile
-            if (HN && pos == slot) fetch_item(f, tbn, IntC<CUR>());
-            if (HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>());
+            if (HN && pos == slot) fetch_item(f, tbn, IntC<CUR>(), pn_c);
+            if (HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>(), pp_c);
           }
           __builtin_amdgcn_sched_barrier(0);
         });
@@ -463,18 +496,21 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // neighbour; the rest is unrolled with the right flags at compile time (KT is a constant).
   // tiles_ahead(T): how many tiles behind tile T+1 have been issued when tile T reaches its barrier
   // (the prologue issued tiles 0..NST-1, tile t issues or completes the issue of tile t-1+NST)
-  tile(0, IntC<0>(), BoolC<(1 < KT)>(), BoolC<(NST < KT)>(), BoolC<false>(), IntC<tiles_ahead(0)>());
-  constexpr int NFULL = KT - NST - 1 > 0 ? KT - NST - 1 : 0;   // tiles 1 .. KT-NST-1 have kt+NST < KT
+  typedef BoolC<false> No;
+  tile(0, IntC<0>(), BoolC<(1 < KTT)>(), BoolC<(NST < KTT)>(), No(), IntC<tiles_ahead(0)>(), IntC<SPW>(),
+       BoolC<(KR > 0 && NST == KT)>(), No());
+  constexpr int NFULL = KT - NST - 1 > 0 ? KT - NST - 1 : 0;   // tiles 1 .. KT-NST-1 have kt+NST < KT: full tiles all round
   constexpr int NG = NFULL / NST;
   for (int g = 0; g < NG; ++g) {
     static_for<0, NST>([&](auto sc) {
       constexpr int S = decltype(sc)::value;
-      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>());
+      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>(), IntC<SPW>(), No(), No());
     });
   }
-  static_for<1 + NG * NST, KT>([&](auto tc) {
+  static_for<1 + NG * NST, KTT>([&](auto tc) {
     constexpr int T = decltype(tc)::value;
-    tile(T, IntC<T % NST>(), BoolC<(T + 1 < KT)>(), BoolC<(T + NST < KT)>(), BoolC<(T - 1 + NST < KT)>(), IntC<tiles_ahead(T)>());
+    tile(T, IntC<T % NST>(), BoolC<(T + 1 < KTT)>(), BoolC<(T + NST < KTT)>(), BoolC<(T - 1 + NST < KTT)>(), IntC<tiles_ahead(T)>(),
+         IntC<(T < KT ? SPW : SPWT)>(), BoolC<(KR > 0 && T + NST == KT)>(), BoolC<(KR > 0 && T - 1 + NST == KT)>());
   });
 
   // the last matrix-core results must have left the pipeline before the epilogue reads them (the
@@ -497,7 +533,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-        gstore<TC, float, 4, false, true>(Cm, v, row, col, N, M, N);
+        gstore<TC, float, 4, (EDGE_M || EDGE_N), true>(Cm, v, row, col, N, M, N);
       }
 }
 

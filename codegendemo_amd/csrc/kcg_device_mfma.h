@@ -199,8 +199,10 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
       auto tile = [&](int kt, auto has1, auto has2) {
         constexpr bool H1 = decltype(has1)::value, H2 = decltype(has2)::value;
         const int cur = kt & 1;
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) {
+        // the step number is a compile-time constant (static_for, not a loop the compiler may decline to
+        // unroll): it selects the half of the fragment double buffer
+        static_for<0, SPW>([&](auto s_c) {
+          constexpr int s = decltype(s_c)::value;
 #pragma unroll
           for (int q = 0; q < NM; ++q) {
             const int slot = s * NM + q;
@@ -224,7 +226,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
             }
             __builtin_amdgcn_sched_barrier(0);
           }
-        }
+        });
         if constexpr (SPW % 2 == 1) {   // odd step count: the prefetched fragments sit in slot 1
 #pragma unroll
           for (int i = 0; i < TMI; ++i) fa[0][i] = fa[1][i];
@@ -259,11 +261,11 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
       if constexpr (C::REGP) {
         Frag fa[2][TMI], fb[2][TNI];
         load_frag(0, wz, fa[0], fb[0]);
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) {
-          if (s + 1 < SPW) load_frag(0, (s + 1) * LSU + wz, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+        static_for<0, SPW>([&](auto s_c) {
+          constexpr int s = decltype(s_c)::value;
+          if constexpr (s + 1 < SPW) load_frag(0, (s + 1) * LSU + wz, fa[(s + 1) & 1], fb[(s + 1) & 1]);
           mma_frag(fa[s & 1], fb[s & 1]);
-        }
+        });
       } else {
         Frag fa[TMI], fb[TNI];
 #pragma unroll

@@ -129,13 +129,20 @@ __device__ __forceinline__ void gemm_simt(const typename C::TA* __restrict__ A, 
   constexpr int KSTEPS = BK / LSU;   // k values of one tile handled by this thread-z slice
   auto compute_tile = [&](int stage) {
     if constexpr (C::REGP) {
-      TA ra[2][TM];
-      TB rb[2][TN];
-      load_frag(stage, tz, ra[0], rb[0]);
+      // two k-steps per iteration with the two fragment buffers named explicitly: the compiler stops
+      // unrolling very large bodies (TM*TN*BK beyond ~16k instructions), and a buffer chosen by a loop
+      // counter that is no longer a constant would turn the register arrays into select chains
+      TA ra0[TM], ra1[TM];
+      TB rb0[TN], rb1[TN];
+      load_frag(stage, tz, ra0, rb0);
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) {
-        if (s + 1 < KSTEPS) load_frag(stage, (s + 1) * LSU + tz, ra[(s + 1) & 1], rb[(s + 1) & 1]);
-        fma_frag(ra[s & 1], rb[s & 1]);
+      for (int s = 0; s < KSTEPS; s += 2) {
+        if (s + 1 < KSTEPS) load_frag(stage, (s + 1) * LSU + tz, ra1, rb1);
+        fma_frag(ra0, rb0);
+        if (s + 1 < KSTEPS) {
+          if (s + 2 < KSTEPS) load_frag(stage, (s + 2) * LSU + tz, ra0, rb0);
+          fma_frag(ra1, rb1);
+        }
       }
     } else {
       TA ra[TM];

@@ -22,6 +22,8 @@ def _exact_case(oracle, cfg, kind, tag):
     print(f"[case] {tag} kind={kind} {M}x{N}x{K} cfg={ {k: cfg[k] for k in ('BLOCK_SIZE_M','BLOCK_SIZE_N','BLOCK_SIZE_K','THREAD_SIZE_M','THREAD_SIZE_N','LOCAL_SPLIT_U','IS_ATRANS','SHARED_PREFETCH','REG_PREFETCH','LOAD_CONTINUOUS','DATATYPE_A')} }", flush=True)
     got, info = run_gemm(cfg, a, b, kind)
     assert info["kind"] == kind
+    if "direct" in tag and kind == MFMA:
+        assert info["lds_bytes"] == 0, "expected the direct-staging kernel (static LDS)"
     want = oracle.matmul(a, b, a_trans=False)
     assert not np.isnan(got).any(), "some C elements were never written"
     bad = np.argwhere(got != want)
@@ -88,6 +90,24 @@ EXACT_CASES = [
                                       shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-1wave", MFMA, dict(M=256, N=256, K=1056, BM=128, BN=128, TM=16, TN=16, BK=32, is_atrans=0,
                                     shared_prefetch=1, reg_prefetch=1)),
+    # direct staging with edge tiles: a partial last K tile (fetched by tile KT-NST, by tile 0, or in the
+    # prologue), rows and columns beyond M and N, both A layouts, both matrix-core tile sizes
+    ("f32-direct-ktail", MFMA, dict(M=256, N=256, K=1000, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=0,
+                                    shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-ktail-bk32-at1", MFMA, dict(M=256, N=256, K=1000, BM=128, BN=128, TM=8, TN=8, BK=32, is_atrans=1,
+                                             shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-ktail-tile0", MFMA, dict(M=256, N=256, K=72, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=0,
+                                          shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-ktail-prologue-at1", MFMA, dict(M=256, N=256, K=24, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=1,
+                                                 shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-edge-mn", MFMA, dict(M=200, N=136, K=104, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=0,
+                                      shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-edge-mn-at1", MFMA, dict(M=200, N=136, K=104, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=1,
+                                          shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-edge-256", MFMA, dict(M=260, N=516, K=1064, BM=256, BN=256, TM=16, TN=16, BK=32, is_atrans=0,
+                                       shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-mf16-ktail", MFMA, dict(M=252, N=248, K=560, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=0,
+                                         shared_prefetch=1, reg_prefetch=1)),
     # fp64 on the matrix cores (16x16x4 instructions, two k values per 16-byte chunk)
     ("mfma-f64", MFMA, dict(M=256, N=256, K=128, dtype=8, scatter=2)),
     ("mfma-f64-at0-both", MFMA, dict(M=256, N=192, K=136, dtype=8, scatter=2, is_atrans=0, shared_prefetch=1,
@@ -159,6 +179,15 @@ HALF_CASES = [
     # one wave per block: 32 fetch instructions per wave and tile limit the number of stages in flight
     ("f16-direct-1wave", dict(M=256, N=256, K=1088, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=16, TN=16,
                               BK=64, shared_prefetch=1, reg_prefetch=1)),
+    # edge tiles through the direct-staging kernel: partial last K tile, rows/columns beyond M and N
+    ("f16-direct-ktail", dict(M=256, N=256, K=992, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
+                              shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-edge-at1", dict(M=200, N=136, K=160, dtype=2, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8,
+                                 BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-direct-256-edge", dict(M=264, N=520, K=1120, dtype=3, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=16, TN=16,
+                                  BK=64, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-edge-out16", dict(M=200, N=136, K=96, dtype=2, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
+                                   shared_prefetch=1, reg_prefetch=1)),
     ("bf16-at0", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=0, BK=32)),
     ("bf16-at1-lsu2", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=1, BK=64, lsu=2)),
 ]
@@ -177,6 +206,8 @@ def test_exact_small_integers_16bit(oracle, tag, kw, kind):
     print(f"[case] {tag} kind={kind} {M}x{N}x{K}", flush=True)
     got, info = run_gemm(cfg, a, b, kind)
     assert info["kind"] == kind
+    if "direct" in tag and kind == MFMA:
+        assert info["lds_bytes"] == 0, "expected the direct-staging kernel (static LDS)"
     want = oracle.matmul(a, b, a_trans=False)
     assert not np.isnan(got).any()
     bad = np.argwhere(got != want)
@@ -201,6 +232,8 @@ def extra_build_configs():
 
 CONFIG4_KERNELS = ((MFMA, dict(BM=128, BN=128, TM=8, TN=8, BK=16, shared_prefetch=1, is_atrans=0)),
                    (MFMA, dict(BM=64, BN=64, BK=32, is_atrans=1)),
+                   # direct staging with a partial last K tile (1000 = 62*16 + 8)
+                   (MFMA, dict(BM=128, BN=64, TM=8, TN=4, BK=16, shared_prefetch=1, reg_prefetch=1, is_atrans=0)),
                    (SIMT, dict(BM=64, BN=64, BK=8, is_atrans=0)))
 CONFIG5_KERNELS = (dict(BM=128, BN=128, TM=8, TN=8, BK=32, shared_prefetch=1, reg_prefetch=1),
                    dict(BM=64, BN=64, BK=32))
