@@ -17,6 +17,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cerrno>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -114,7 +115,10 @@ struct RtcApi {
 void* open_shared(const char* soname, std::string* err) {
   void* h = dlopen(soname, RTLD_NOW | RTLD_NOLOAD);
   if (!h) h = dlopen(soname, RTLD_NOW | RTLD_LOCAL);
-  if (!h && err) *err = std::string("cannot load ") + soname + ": " + (dlerror() ? dlerror() : "?");
+  if (!h && err) {
+    const char* why = dlerror();   // one call: it clears the message it returns
+    *err = std::string("cannot load ") + soname + ": " + (why ? why : "?");
+  }
   return h;
 }
 
@@ -580,7 +584,13 @@ int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[
   hipEvent_t e0, e1;
   HIP_READY();
   HIP_TRY(HIPF(hipEventCreate)(&e0));
-  HIP_TRY(HIPF(hipEventCreate)(&e1));
+  {
+    hipError_t e = HIPF(hipEventCreate)(&e1);
+    if (e != hipSuccess) {
+      (void)HIPF(hipEventDestroy)(e0);
+      return hip_fail(e, "hipEventCreate");
+    }
+  }
   int rc = KCG_OK;
   std::vector<float> samples;
   auto timed = [&](int n, float* ms) -> int {
