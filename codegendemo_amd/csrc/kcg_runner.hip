@@ -18,6 +18,11 @@
 //       instruction shapes and for operands of all zeros and of normal(0, 0.5) values.  On a
 //       power-limited part the second figure is the ceiling of any GEMM on such data.
 //
+//   kcg_runner --launch-cost
+//       the fixed costs a short GEMM pays per launch on this GPU: the period of back-to-back launches of
+//       an empty kernel (1 block; 256 blocks; 256 blocks with 64 KiB of LDS each) and of a kernel that
+//       only writes 64 MiB (the fp32 result of a 4096 x 4096 product)
+//
 // Build: make -C codegendemo_amd/csrc runner      (hipcc --offload-arch=gfx950)
 #include <hip/hip_runtime.h>
 
@@ -186,6 +191,53 @@ static int mfma_peak_main(const char* tname) {
   return 0;
 }
 
+// ---- fixed costs of a launch: what a GEMM of a few hundred microseconds pays besides its K loop ------
+__global__ void empty_kernel(float* sink) {
+  if (sink == nullptr && threadIdx.x == 12345) *sink = 0.f;   // never true
+}
+template <int LDS_BYTES>
+__global__ __launch_bounds__(256) void empty_kernel_lds(float* sink) {
+  __shared__ char big[LDS_BYTES];
+  if (sink == nullptr) { big[threadIdx.x] = 1; *sink = big[255 - threadIdx.x]; }   // never true; keeps the array
+}
+// every block writes its own contiguous piece of `out` with 16-byte stores, nothing else
+__global__ __launch_bounds__(256) void write_only(float4* __restrict__ out, size_t per_block) {
+  float4* p = out + (size_t)blockIdx.x * per_block;
+  const float4 v = {1.f, 2.f, 3.f, 4.f};
+  for (size_t i = threadIdx.x; i < per_block; i += 256) p[i] = v;
+}
+
+template <class F>
+static double launch_period_us(F launch, int n) {
+  for (int i = 0; i < 200; ++i) launch();
+  hipEvent_t e0, e1;
+  HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+  HIP_OK(hipEventRecord(e0, 0));
+  for (int i = 0; i < n; ++i) launch();
+  HIP_OK(hipEventRecord(e1, 0));
+  HIP_OK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1));
+  return ms * 1e3 / n;
+}
+
+static int launch_cost_main() {
+  float* sink;
+  const size_t bytes = (size_t)64 << 20;   // the C matrix of a 4096 x 4096 fp32 result
+  HIP_OK(hipMalloc(&sink, bytes));
+  const int n = 2000;
+  const double e1 = launch_period_us([&] { hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, 0, sink); }, n);
+  const double e256 = launch_period_us([&] { hipLaunchKernelGGL(empty_kernel, dim3(256), dim3(256), 0, 0, sink); }, n);
+  const double elds = launch_period_us([&] { hipLaunchKernelGGL((empty_kernel_lds<65536>), dim3(256), dim3(256), 0, 0, sink); }, n);
+  const double w = launch_period_us([&] { hipLaunchKernelGGL(write_only, dim3(256), dim3(256), 0, 0, (float4*)sink, bytes / 16 / 256); }, 500);
+  printf("{\"launch_cost\": {\"period_us\": {\"empty_1_block\": %.2f, \"empty_256_blocks\": %.2f, \"empty_256_blocks_64KiB_lds\": %.2f, "
+         "\"write_64MiB\": %.2f}, \"write_GBps\": %.0f, \"note\": \"back-to-back launches on one stream, HIP events around the whole run\"}}\n",
+         e1, e256, elds, w, bytes / (w - e256) * 1e-3);
+  HIP_OK(hipFree(sink));
+  return 0;
+}
+
 static float lcg_uniform(uint64_t& s) {   // [-1, 1)
   s = s * 6364136223846793005ull + 1442695040888963407ull;
   return (float)((int32_t)(s >> 40) - (1 << 23)) / (float)(1 << 23);
@@ -246,6 +298,7 @@ int main(int argc, char** argv) {
     if (argc >= 3 && !strcmp(argv[2], "bf16")) return mfma_peak_main<b8_t, __bf16>("bf16");
     return mfma_peak_main<h8_t, _Float16>("f16");
   }
+  if (argc >= 2 && !strcmp(argv[1], "--launch-cost")) return launch_cost_main();
   if (argc >= 3 && !strcmp(argv[1], "--config")) {
     std::string path = argv[2];
     for (int i = 3; i + 1 < argc; i += 2) {

@@ -68,3 +68,15 @@ def test_runner_mfma_peak_mode():
     r = json.loads(p.stdout.strip().splitlines()[-1])["mfma_peak"]
     for shape in ("16x16x32", "32x32x16"):
         assert 500.0 < r["normal(0,0.5)"][shape] <= r["zeros"][shape] * 1.02 < 2516.6 * 1.05
+
+
+def test_runner_launch_cost_mode():
+    """Fixed costs per launch: an empty kernel's back-to-back period is a few microseconds, and writing
+    64 MiB (the fp32 result of a 4096 x 4096 product) cannot beat the 8 TB/s of HBM."""
+    p = _run(["--launch-cost"])
+    assert p.returncode == 0
+    r = json.loads(p.stdout.strip().splitlines()[-1])["launch_cost"]
+    per = r["period_us"]
+    assert 0.5 < per["empty_1_block"] < 50.0 and 0.5 < per["empty_256_blocks"] < 50.0
+    assert per["write_64MiB"] > per["empty_256_blocks"] + (64 << 20) / 8e12 * 1e6
+    assert 1000.0 < r["write_GBps"] < 8000.0
