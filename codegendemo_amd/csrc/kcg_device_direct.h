@@ -349,6 +349,16 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // lgkmcnt(0): every LDS read issued so far has returned
   auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
 
+  // prologue, first half: the first NST tiles go out together (the wait further down is for tile 0
+  // alone: its successors' memory latency overlaps with it instead of following it), and before
+  // anything else that takes time: clearing the accumulators runs under that latency
+  static_for<0, NST>([&](auto t) {
+    if (decltype(t)::value < KTT) {
+#pragma unroll
+      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t, BoolC<(KR > 0 && decltype(t)::value == KT)>());
+    }
+  });
+
   Acc acc[TMI][TNI];
 #pragma unroll
   for (int i = 0; i < TMI; ++i)
@@ -398,17 +408,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     return cmax(0, last - (t + 1));
   };
 
-  // prologue: tile 0 -> stage 0, wait for it; then tiles 1..NST-1 in flight
-#pragma unroll
-  for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(0), IntC<0>(), BoolC<false>());
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's chunks of tile 0 are in LDS
-  __syncthreads();
-  static_for<1, NST>([&](auto t) {
-    if (decltype(t)::value < KTT) {
-#pragma unroll
-      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t, BoolC<(KR > 0 && decltype(t)::value == KT)>());
-    }
-  });
+  // prologue, second half
+  constexpr int NPRO = cmin(NST, KTT);                                    // tiles the prologue has issued
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(cmin(63, (NPRO - 1) * NFETCH)));  // this wave's chunks of tile 0 are in LDS
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();                                            // ... and everyone's (bare barrier: see the K loop)
+  asm volatile("" ::: "memory");
   FragA fa[TMI];
   FragB fb[2][TNI];
   static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
