@@ -16,7 +16,8 @@
 //       what the matrix pipeline of this GPU sustains with nothing else going on: a loop of independent
 //       matrix-core instructions on register operands, timed over ~0.3 s per case, for both 16-bit
 //       instruction shapes and for operands of all zeros and of normal(0, 0.5) values.  On a
-//       power-limited part the second figure is the ceiling of any GEMM on such data.
+//       power-limited part the second figure is the ceiling of any GEMM on such data.  Also prints how long
+//       the blocks of each of the eight XCDs took in the last launch (the XCDs do not run at one clock).
 //
 //   kcg_runner --launch-cost
 //       the fixed costs a short GEMM pays per launch on this GPU: the period of back-to-back launches of
@@ -94,7 +95,8 @@ template <> struct PeakOp<b8_t> {
 // opnd: 32 fragments of 8 values per lane (65536 lanes).  SMALL: 8x8 tiles of 16x16x32 over two k-steps;
 // otherwise 4x4 tiles of 32x32x16 over four k-steps: 2^22 flop per lane-iteration either way.
 template <class V, bool SMALL>
-__global__ __launch_bounds__(256) void mfma_peak(const V* __restrict__ opnd, float* sink, int iters) {
+__global__ __launch_bounds__(256) void mfma_peak(const V* __restrict__ opnd, float* sink, int iters, long long* ticks) {
+  const long long t_begin = __builtin_amdgcn_s_memrealtime();   // 100 MHz
   const int tid = blockIdx.x * 256 + threadIdx.x;
   V frag[32];
 #pragma unroll
@@ -140,20 +142,35 @@ __global__ __launch_bounds__(256) void mfma_peak(const V* __restrict__ opnd, flo
       for (int j = 0; j < 4; ++j) s += acc[i][j][0] + acc[i][j][15];
   }
   if (s == 1234.5f) sink[tid] = s;   // keeps the loop alive; practically never true
+  if (ticks && threadIdx.x == 0) ticks[blockIdx.x] = __builtin_amdgcn_s_memrealtime() - t_begin;
 }
 
+// xcd_ns (optional, 8 values): mean block duration of the last launch per XCD (blocks are dealt to the
+// eight XCDs round-robin), in nanoseconds
 template <class V, bool SMALL>
-static double run_mfma_peak(const V* d_opnd, float* d_sink) {
+static double run_mfma_peak(const V* d_opnd, float* d_sink, double* xcd_ns = nullptr) {
   const int iters = 3000, launches = 50;           // 64 (or 4x16) instructions of 2^22/64 flop per lane-iteration
-  for (int i = 0; i < launches; ++i) hipLaunchKernelGGL((mfma_peak<V, SMALL>), dim3(256), dim3(256), 0, 0, d_opnd, d_sink, iters);
+  long long* d_ticks;
+  HIP_OK(hipMalloc(&d_ticks, 256 * sizeof(long long)));
+  for (int i = 0; i < launches; ++i) hipLaunchKernelGGL((mfma_peak<V, SMALL>), dim3(256), dim3(256), 0, 0, d_opnd, d_sink, iters, d_ticks);
   hipEvent_t e0, e1;
   HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
   HIP_OK(hipEventRecord(e0, 0));
-  for (int i = 0; i < launches; ++i) hipLaunchKernelGGL((mfma_peak<V, SMALL>), dim3(256), dim3(256), 0, 0, d_opnd, d_sink, iters);
+  for (int i = 0; i < launches; ++i) hipLaunchKernelGGL((mfma_peak<V, SMALL>), dim3(256), dim3(256), 0, 0, d_opnd, d_sink, iters, d_ticks);
   HIP_OK(hipEventRecord(e1, 0));
   HIP_OK(hipEventSynchronize(e1));
   float ms = 0.f;
   HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  if (xcd_ns) {
+    long long h[256];
+    HIP_OK(hipMemcpy(h, d_ticks, sizeof(h), hipMemcpyDeviceToHost));
+    for (int x = 0; x < 8; ++x) {
+      double sum = 0;
+      for (int b = x; b < 256; b += 8) sum += (double)h[b] * 10.0;
+      xcd_ns[x] = sum / 32;
+    }
+  }
+  HIP_OK(hipFree(d_ticks));
   const double flops = (double)launches * iters * 128.0 * 16 * 16 * 32 * 2 * 4 * 256;   // per block: 4 waves
   return flops / (ms * 1e-3) / 1e12;
 }
@@ -182,8 +199,11 @@ static int mfma_peak_main(const char* tname) {
         h[i][e] = (E)g;
       }
     HIP_OK(hipMemcpy(d, h.data(), n * sizeof(V), hipMemcpyHostToDevice));
-    const double small = run_mfma_peak<V, true>(d, sink), big = run_mfma_peak<V, false>(d, sink);
-    printf(", \"%s\": {\"16x16x32\": %.1f, \"32x32x16\": %.1f}", pass == 0 ? "zeros" : "normal(0,0.5)", small, big);
+    double xcd[8];
+    const double small = run_mfma_peak<V, true>(d, sink, xcd), big = run_mfma_peak<V, false>(d, sink);
+    printf(", \"%s\": {\"16x16x32\": %.1f, \"32x32x16\": %.1f, \"16x16x32_block_us_by_xcd\": [", pass == 0 ? "zeros" : "normal(0,0.5)", small, big);
+    for (int x = 0; x < 8; ++x) printf("%s%.1f", x ? ", " : "", xcd[x] * 1e-3);
+    printf("]}");
   }
   printf(", \"unit\": \"TFLOP/s\"}}\n");
   HIP_OK(hipFree(d));
