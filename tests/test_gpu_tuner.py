@@ -60,3 +60,13 @@ def test_perf_tester_fp16_in_process(tmp_path, monkeypatch):
     PerfTester._a = PerfTester._b = PerfTester._aT = None
     PerfTester.D = None
     PerfTester.torch_eps = 0.0
+
+
+@pytest.mark.parametrize("case", ["case_normal_0", "case_normal_1"])
+def test_single_config_check_script(case, capsys):
+    """python -m codegendemo_amd.kcg.test <case>: compile, one run, allclose(1e-2) against torch.matmul."""
+    from codegendemo_amd.kcg import test as single
+    print(f"[case] single-config check {case}", flush=True)
+    assert single.main([case]) == 0
+    out = capsys.readouterr().out
+    assert "test correct!" in out and "speed up:" in out and "kernelName =  GEMM_MNK1024x" in out

@@ -173,3 +173,17 @@ def test_uniform_stream_golden_values():
     assert got == want["raw_bits_stream1_first4"]
     assert SI.checksum(SI.uniform((256, 256), SI.STREAM_A)) == want["checksum_uniform_256x256_stream1"]
     assert SI.checksum(SI.uniform((256, 256), SI.STREAM_B)) == want["checksum_uniform_256x256_stream2"]
+
+
+def test_single_config_check_cases(capsys):
+    """The hand-written cases of the reference's test.py (:19-107): the two normal ones are valid configs
+    with the launch geometry its comments state; the 'bad' one is refused before anything is compiled."""
+    from codegendemo_amd.kcg import test as single
+    k0 = single.make_case("case_normal_0")
+    k0.check()
+    assert (k0.M, k0.N, k0.K, k0.LOCAL_SPLIT_U, k0.isATranspose) == (1024, 1056, 1024, 2, 1)
+    grid, block = _native.launch_dims(k0.values())
+    assert grid[0] == 16 * 22 and block[0] == 256            # matmul.cpp:2448-2449
+    single.make_case("case_normal_1").check()
+    assert single.main(["case_bad_0"]) == 2
+    assert "invalid config" in capsys.readouterr().out
