@@ -1,72 +1,50 @@
-"""CompiledKernel: a loaded (lazily) and launchable GEMM kernel.
-
-Counterpart of Runtime/python/kcg/CompiledKernel.py (:6-23) with the loader (Loader.py:64-105,
-loaderCCode/hip.c:60-133) and launcher (HIPLauncher.py:264-314) folded in: the reference gcc-built a
-loader extension and a per-signature launch stub at run time; here both are entry points of
-libkcg_gemm.so.  Instances are picklable before their first run and load the code object in the
-process that first launches them (they cross a process boundary in a .pkl, KCGTask.py:305-318).
-"""
-from .. import _native
-
-
-def _device_address(x):
-    """int, None, or anything with .data_ptr() (HIPLauncher.py:148-187)."""
-    if x is None:
-        return 0
-    if isinstance(x, int):
-        return x
-    return int(x.data_ptr())
+"""CompiledKernel: a lazily loaded, launchable GEMM kernel (reference: Runtime/python/kcg/CompiledKernel.py:6-23):
+a HIPLauncher around a KernelLibFile, loaded by the HIPLoaderST singleton on first use.  Instances are
+picklable before and after their first run: handles stay in the process that loaded them, and the
+process that unpickles loads the code object again (they cross a process boundary in a .pkl,
+KCGTask.py:305-318)."""
+from .HIPLauncher import HIPLauncher
+from .Loader import HIPLoaderST
 
 
 class CompiledKernel:
     def __init__(self, kernelBinaryPath: str, kernelName: str, shmSize: int, kernel_signature,
                  gridDims: list, blockDims: list, device=0):
-        self.kernelBinaryPath = kernelBinaryPath
-        self.kernelName = kernelName
-        self.shmSize = int(shmSize)
         self.signature = kernel_signature
-        self.gridDims = [int(x) for x in gridDims]
-        self.blockDims = [int(x) for x in blockDims]
         self.device = int(device)
-        self._module = 0
-        self._function = 0
-        self.n_regs = None
-        self.n_spills = None
+        self.m_loader = HIPLoaderST()
+        self.m_launcher = HIPLauncher(kernelBinaryPath, kernelName, shmSize, self.signature, gridDims, blockDims, device)
 
-    # ---- pickling: handles are per process ----------------------------------------------------
+    # the launcher's view, under the names the rest of the package and its users read
+    kernelBinaryPath = property(lambda self: self.m_launcher.m_kernelLib.m_filePath)
+    kernelName = property(lambda self: self.m_launcher.m_kernelLib.m_kernelFuncName)
+    shmSize = property(lambda self: self.m_launcher.m_kernelLib.m_shmSize)
+    gridDims = property(lambda self: self.m_launcher.m_kernelLib.m_gridDims)
+    blockDims = property(lambda self: self.m_launcher.m_kernelLib.m_blockDims)
+
+    def _info(self):
+        return self.m_loader.loadBinary(self.m_launcher.m_kernelLib)
+
+    n_regs = property(lambda self: self._info().m_nRegs)
+    n_spills = property(lambda self: self._info().m_nSpills)
+
     def __getstate__(self):
         st = dict(self.__dict__)
-        st["_module"] = 0
-        st["_function"] = 0
+        st.pop("m_loader", None)            # a per-process singleton
         return st
 
-    def _ensure_loaded(self):
-        if not self._function:
-            self._module, self._function, self.n_regs, self.n_spills = _native.load(
-                self.kernelBinaryPath, self.kernelName, self.shmSize, self.device)
-        return self._function
-
-    def _stream(self):
-        import torch
-        return torch.cuda.current_stream(self.device).cuda_stream
+    def __setstate__(self, st):
+        self.__dict__.update(st)
+        self.m_loader = HIPLoaderST()
 
     def run(self, *args, **kwargs):
         """Launch on torch's current stream of this kernel's device with (a, b, c)."""
-        if len(args) != 3:
-            raise TypeError(f"GEMM kernel takes 3 device buffers (a, b, c), got {len(args)}")
-        fn = self._ensure_loaded()
-        a, b, c = (_device_address(x) for x in args)
-        _native.launch(fn, self.gridDims, self.blockDims, self.shmSize, self._stream(), a, b, c)
+        if self.m_launcher is not None:
+            self.m_launcher.launchKernel(self.device, *args)
 
     def benchmark(self, a, b, c, warmup=1, iters=20, reps=0):
         """HIP-event timing in C: (median_ms, min_ms) per launch."""
-        fn = self._ensure_loaded()
-        a, b, c = (_device_address(x) for x in (a, b, c))
-        return _native.benchmark(fn, self.gridDims, self.blockDims, self.shmSize, self._stream(), a, b, c,
-                                 warmup, iters, reps)
+        return self.m_launcher.benchmarkKernel(self.device, a, b, c, warmup, iters, reps)
 
     def unload(self):
-        if self._module:
-            _native.unload(self._module)
-        self._module = 0
-        self._function = 0
+        self.m_loader.unloadBinary(self.m_launcher.m_kernelLib)

@@ -87,11 +87,39 @@ def test_compiler_return_shape_and_factory(tmp_path, monkeypatch):
     kernel = CompiledKernelFactory.getKernel(ui, 0)
     assert kernel.signature == {0: "*fp32", 1: "*fp32", 2: "*fp32"}
     # picklable before first run, handles never travel (KCGTask.py:305-318)
-    kernel._module, kernel._function = 11, 22
+    from codegendemo_amd.kcg.Kernel import EnumBackendType, KernelRuntimeInfo
+    from codegendemo_amd.kcg.Loader import HIPLoaderST
+    lib = kernel.m_launcher.m_kernelLib                     # KernelLibFile (Kernel.py:52-71)
+    assert lib.m_backendType == EnumBackendType.HIP and lib.m_shmSize == ui.sharedMem() and lib.m_device == 0
+    assert lib.signature_str() == "*fp32*fp32*fp32" and len(lib.hash()) == 10
+    assert kernel.m_loader is HIPLoaderST() and HIPLoaderST() is HIPLoaderST()      # per-process singleton
+    lib.m_kernelInfo = KernelRuntimeInfo(11, 22, 0, 0)
     k2 = pickle.loads(pickle.dumps((kpm, ui, kernel)))[2]
-    assert k2._function == 0 and k2.kernelBinaryPath == path and k2.gridDims == [256, 1, 1]
+    assert k2.m_launcher.m_kernelLib.m_kernelInfo is None and k2.m_loader is HIPLoaderST()
+    assert k2.kernelBinaryPath == path and k2.gridDims == [256, 1, 1] and k2.kernelName == name
+    lib.m_kernelInfo = None
     with pytest.raises(TypeError):
         k2.run(1, 2)
+
+
+def test_launcher_refuses_operands_smaller_than_the_kernel_accesses(tmp_path, monkeypatch):
+    """The kernel name carries M, N, K and the element types: a tensor with fewer bytes than the kernel
+    will touch is refused on the host (on the device it would be a memory fault)."""
+    import torch
+    from codegendemo_amd.kcg.HIPLauncher import HIPLauncher
+    from codegendemo_amd.kcg.Kernel import operand_bytes
+    name = _native.kernel_name(kernelArgFromConfig(make_config(512, 256, 128, dtype=2, dtype_c=4)).values())
+    assert operand_bytes(name) == (512 * 128 * 2, 128 * 256 * 2, 512 * 256 * 4)
+    assert operand_bytes("some_other_kernel") is None
+    launcher = HIPLauncher(str(tmp_path / "missing.hsaco"), name, 0, {}, [8, 1, 1], [256, 1, 1], 0)
+    a = torch.zeros(512, 128, dtype=torch.float16)
+    b = torch.zeros(128, 256, dtype=torch.float16)
+    with pytest.raises(ValueError, match="operand c: .* accesses 524288 bytes"):
+        launcher.launchKernel(0, a, b, torch.zeros(512, 256, dtype=torch.float16))
+    with pytest.raises(ValueError, match="operand a must be contiguous"):
+        launcher.launchKernel(0, torch.zeros(128, 512, dtype=torch.float16).t(), b, torch.zeros(512, 256))
+    with pytest.raises(_native.KcgError):                   # sizes fine: it gets as far as the (missing) code object
+        launcher.launchKernel(0, a, b, torch.zeros(512, 256))
 
 
 def test_tuning_space_checkers():

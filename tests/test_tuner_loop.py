@@ -60,7 +60,7 @@ def test_compile_task_writes_pickle(workdir):
     assert pkls == ["valid_kernels_unit_0_3.pkl"]
     back = deserialize_from_file(os.path.join(PathManager.pikle_dir(), pkls[0]))
     assert [t[0].BLOCK_SIZE_K for t in back] == [16, 32]
-    assert back[0][2]._function == 0 and back[0][1].sharedMem() == back[0][2].shmSize
+    assert back[0][2].m_launcher.m_kernelLib.m_kernelInfo is None and back[0][1].sharedMem() == back[0][2].shmSize
     # a truncated pickle reads as "no kernels" (Utils.py:44-51)
     p = os.path.join(PathManager.pikle_dir(), "broken.pkl")
     with open(p, "wb") as f:
