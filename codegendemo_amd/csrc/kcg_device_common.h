@@ -14,12 +14,16 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// Raw 1..16-byte carriers for copy_bytes.  They are declared may_alias: copy_bytes moves floats, halves
+// and doubles through them, and without the attribute the compiler is entitled to assume that a store
+// through `unsigned int` cannot change a `float` object (type-based alias analysis) and to reorder the
+// typed accesses around the copy.
 template <int BYTES> struct RawVec;
 template <> struct RawVec<1> { typedef unsigned char type; };
-template <> struct RawVec<2> { typedef unsigned short type; };
-template <> struct RawVec<4> { typedef unsigned int type; };
-template <> struct RawVec<8> { typedef u32x2 type; };
-template <> struct RawVec<16> { typedef u32x4 type; };
+template <> struct RawVec<2> { typedef unsigned short __attribute__((may_alias)) type; };
+template <> struct RawVec<4> { typedef unsigned int __attribute__((may_alias)) type; };
+template <> struct RawVec<8> { typedef u32x2 __attribute__((may_alias)) type; };
+template <> struct RawVec<16> { typedef u32x4 __attribute__((may_alias)) type; };
 
 template <class T> struct AccOf { typedef float type; };
 template <> struct AccOf<double> { typedef double type; };
@@ -137,18 +141,18 @@ __device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r,
       for (int e = 0; e < VEC; ++e) dst[e] = base[(long)r * LD + c + e];
     }
   } else if constexpr (ALIGNED) {
-    // c and CMAX are multiples of VEC: the vector lies inside or outside as a whole (one predicate per
-    // vector instead of one per element)
-    if (r < RMAX && c < CMAX) {
-      copy_bytes<VEC * (int)sizeof(T)>(dst, base + (long)r * LD + c);
-    } else {
+    // c and CMAX are multiples of VEC: the vector lies inside or outside as a whole.  No branch: a lane
+    // whose vector lies outside loads element 0 of the matrix instead and then drops it.
+    const bool in = r < RMAX && c < CMAX;
+    copy_bytes<VEC * (int)sizeof(T)>(dst, base + (in ? (long)r * LD + c : 0L));
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) dst[e] = T(0);
-    }
+    for (int e = 0; e < VEC; ++e) dst[e] = in ? dst[e] : T(0);
   } else {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-      dst[e] = (r < RMAX && c + e < CMAX) ? base[(long)r * LD + c + e] : T(0);
+      const bool in = r < RMAX && c + e < CMAX;
+      const T v = base[in ? (long)r * LD + c + e : 0L];
+      dst[e] = in ? v : T(0);
     }
   }
 }

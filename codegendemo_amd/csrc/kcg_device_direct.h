@@ -521,6 +521,14 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // the last matrix-core results must have left the pipeline before the epilogue reads them (the
   // compiler, which normally inserts these wait states, does not know the instructions above)
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  // ... and the epilogue's reads must stay behind those wait states: an accumulator is an ordinary
+  // register value to the compiler, free to be read (converted, moved) ahead of an asm statement that does
+  // not mention it.  Passing every accumulator through an empty asm statement behind the wait states
+  // makes each read depend on it (asm volatile statements keep their order).
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNI; ++j) asm volatile("" : "+a"(acc[i][j]));
   // ---- epilogue --------------------------------------------------------------------------------
   // With swapped operands a 32x32 accumulator holds, per lane, row m = lane%32 and columns
   // n = 8*g + 4*(lane/32) + {0..3} for g = 0..3 (16x16: row lane%16, columns 4*(lane/16) + {0..3}).

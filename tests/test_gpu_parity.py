@@ -108,6 +108,16 @@ EXACT_CASES = [
                                        shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-mf16-ktail", MFMA, dict(M=252, N=248, K=560, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=0,
                                          shared_prefetch=1, reg_prefetch=1)),
+    # scalar kernel, edge tiles under register pressure (16-wide thread tiles, a one-wave block with 192
+    # staging registers): shapes that returned wrong values while edge loads ran under a branch
+    ("simt-edge-16x8-both", SIMT, dict(M=244, N=376, K=112, BM=128, BN=128, BK=16, TM=16, TN=8, is_atrans=1,
+                                       shared_prefetch=1, reg_prefetch=1, block_mapping=0, reduce_c_continuous=0)),
+    ("simt-edge-1wave-8x16", SIMT, dict(M=124, N=124, K=133, BM=64, BN=128, BK=64, TM=8, TN=16, is_atrans=1,
+                                        shared_prefetch=1, reg_prefetch=1, block_mapping=2, load_continuous=0,
+                                        scatter=2, glw=1)),
+    ("simt-edge-1wave-8x16-glw4", SIMT, dict(M=124, N=124, K=136, BM=64, BN=128, BK=64, TM=8, TN=16, is_atrans=1,
+                                             shared_prefetch=1, reg_prefetch=1, block_mapping=2, load_continuous=0,
+                                             scatter=2, glw=4)),
     # fp64 on the matrix cores (16x16x4 instructions, two k values per 16-byte chunk)
     ("mfma-f64", MFMA, dict(M=256, N=256, K=128, dtype=8, scatter=2)),
     ("mfma-f64-at0-both", MFMA, dict(M=256, N=192, K=136, dtype=8, scatter=2, is_atrans=0, shared_prefetch=1,
@@ -188,6 +198,12 @@ HALF_CASES = [
                                   BK=64, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-edge-out16", dict(M=200, N=136, K=96, dtype=2, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
                                    shared_prefetch=1, reg_prefetch=1)),
+    # 16-bit output behind an edge predicate with 32x32x16 instructions: the epilogue's conversions must not
+    # be scheduled in front of the wait states that follow the last matrix instruction
+    ("bf16-direct-edge-out16-mf32", dict(M=40, N=128, K=48, dtype=3, dtype_c=3, is_atrans=1, BM=64, BN=128, BK=16, TM=8,
+                                         TN=8, shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-edge-out16-mf32-at0", dict(M=48, N=120, K=32, dtype=2, dtype_c=2, is_atrans=0, BM=64, BN=128, BK=16,
+                                            TM=8, TN=8, shared_prefetch=1, reg_prefetch=1)),
     ("bf16-at0", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=0, BK=32)),
     ("bf16-at1-lsu2", dict(M=256, N=256, K=128, dtype=3, dtype_c=4, is_atrans=1, BK=64, lsu=2)),
 ]
