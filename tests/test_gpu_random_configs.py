@@ -1,6 +1,7 @@
-"""A fixed pseudo-random sample of tuning configs (both kernel families, all input types, both A layouts,
-prefetch flags, split-U, odd tile/wave shapes, 1..17 K tiles), each checked bit for bit against the CPU
-oracle on small-integer data.  The sample is deterministic, so the build step can precompile it."""
+"""Two fixed pseudo-random samples of tuning configs (both kernel families, all input types, both A
+layouts, prefetch flags, split-U, odd tile/wave shapes, 1..17 K tiles; the second with edge tiles in M,
+N and K), each checked bit for bit on small-integer data: the first against the CPU oracle, the second
+against the exact integer product.  The samples are deterministic, so the build step can precompile them."""
 import random
 
 import numpy as np
@@ -56,6 +57,96 @@ def random_configs(n_matrix=60, n_simt=30, seed=20240607):
         except (ValueError, _native.KcgError):
             continue
     return out
+
+
+def random_edge_configs(n_matrix=50, n_simt=30, n_direct=25, seed=20250311):
+    """-> [(config, kind)]: a second fixed sample whose shapes are not multiples of the tiles: rows and
+    columns beyond M and N, K remainders (whole k-steps and odd ones), 16-bit outputs, 2..16-wide thread
+    tiles also for the scalar kernel, one-wave blocks, narrow load widths."""
+    rng = random.Random(seed)
+    out = []
+    want = {_native.KIND_MFMA: n_matrix, _native.KIND_SIMT: n_simt}
+    have = {_native.KIND_MFMA: 0, _native.KIND_SIMT: 0}
+    while have != want:
+        kind = rng.choice([_native.KIND_SIMT, _native.KIND_MFMA, _native.KIND_MFMA])
+        if have[kind] == want[kind]:
+            continue
+        dtype = rng.choice([2, 3, 4, 4, 8])
+        g = {2: 8, 3: 8, 4: 4, 8: 2}[dtype]
+        BM, BN = rng.choice([32, 64, 128, 256]), rng.choice([32, 64, 128, 256])
+        BK = rng.choice([8, 16, 32, 64] if dtype in (4, 8) else [16, 32, 64])
+        kw = dict(BM=BM, BN=BN, BK=BK, TM=rng.choice([2, 4, 8, 16]), TN=rng.choice([2, 4, 8, 16]),
+                  warp_layout=rng.choice([(8, 8), (8, 8), (4, 16), (16, 4)]), dtype=dtype, is_atrans=rng.choice([0, 1]),
+                  block_mapping=rng.choice([0, 2, 8]), lsu=rng.choice([1, 1, 1, 2]),
+                  load_continuous=rng.choice([0, 1, 1, 1]), reduce_c_continuous=rng.choice([0, 1]))
+        kw["shared_prefetch"], kw["reg_prefetch"] = rng.choice([(1, 1), (1, 1), (1, 1), (1, 0), (0, 1), (0, 0)])
+        out16 = dtype in (2, 3) and rng.random() < 0.3
+        if dtype in (2, 3):
+            kw["dtype_c"] = dtype if out16 else 4
+        if rng.random() < 0.3:
+            kw["scatter"] = rng.choice([1, 2])
+        if rng.random() < 0.1:
+            kw["glw"] = rng.choice([1, 2])
+        kt = rng.choice([1, 2, 3] if out16 else [1, 2, 3, 4, 5, 7, 9, 12, 17])     # 16-bit sums must stay exact
+        kw.update(M=BM * rng.choice([1, 2]) - rng.choice([0, 0, g, 3 * g, 1, 5, BM - g]),
+                  N=BN * rng.choice([1, 2, 3]) - rng.choice([0, 0, g, 2 * g, 3, BN - g]),
+                  K=BK * kt + rng.choice([0, 0, 8, 16, 32, 4, 24, 2, 1, 5]) % BK)
+        if kw["M"] <= 0 or kw["N"] <= 0:
+            continue
+        try:
+            cfg = make_config(**kw)
+            if _native.is_valid_config(kernelArgFromConfig(cfg).values(), kind):
+                out.append((cfg, kind))
+                have[kind] += 1
+        except (ValueError, _native.KcgError):
+            continue
+    # ... and configs that take the direct-staging kernel with such shapes (K remainders of whole k-steps)
+    n = 0
+    while n < n_direct:
+        dtype = rng.choice([2, 3, 4, 4])
+        g = 4 if dtype == 4 else 8
+        BM, BN = rng.choice([64, 128, 256]), rng.choice([64, 128, 256])
+        BK = rng.choice([8, 16, 32, 64] if dtype == 4 else [16, 32, 64])
+        out16 = dtype != 4 and rng.random() < 0.3
+        kt = rng.choice([1, 2, 3] if out16 else [1, 2, 3, 4, 5, 7, 9, 12, 17])
+        kw = dict(BM=BM, BN=BN, BK=BK, TM=rng.choice([2, 4, 8, 16]), TN=rng.choice([2, 4, 8, 16]),
+                  warp_layout=rng.choice([(8, 8), (8, 8), (4, 16), (16, 4)]), dtype=dtype, is_atrans=rng.choice([0, 1]),
+                  block_mapping=rng.choice([0, 2, 4, 8]), shared_prefetch=1, reg_prefetch=1,
+                  M=BM * rng.choice([1, 2]) - g * rng.choice([0, 1, 3, BM // g - 1, BM // (2 * g)]),
+                  N=BN * rng.choice([1, 2, 3]) - g * rng.choice([0, 1, 2, BN // g - 1, BN // (2 * g)]),
+                  K=BK * kt + rng.choice([0, 8, 16, 32, 48]) % BK)
+        if dtype != 4:
+            kw["dtype_c"] = dtype if out16 else 4
+        if kw["M"] <= 0 or kw["N"] <= 0 or (kw["M"] % BM == 0 and kw["N"] % BN == 0 and kw["K"] % BK == 0):
+            continue
+        try:
+            cfg = make_config(**kw)
+            v = kernelArgFromConfig(cfg).values()
+            if _native.is_valid_config(v, _native.KIND_MFMA) and \
+                    "DIRECT = true" in _native.instantiation_source(v, _native.KIND_MFMA):
+                out.append((cfg, _native.KIND_MFMA))
+                n += 1
+        except (ValueError, _native.KcgError):
+            continue
+    return out
+
+
+def test_random_edge_config_sample_is_bit_exact():
+    """Entries in {-1, 0, 1}: every sum is an integer of magnitude <= K, exact in fp32 and, for the 16-bit
+    outputs (K <= 255 there), in fp16 and bf16 as well."""
+    cases = random_edge_configs()
+    direct = 0
+    for i, (cfg, kind) in enumerate(cases):
+        M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+        a = SI.small_ints((M, K), SI.STREAM_A, lim=1)
+        b = SI.small_ints((K, N), SI.STREAM_B, lim=1)
+        print(f"[case] random edge {i} kind={kind} {kernelArgFromConfig(cfg).values()}", flush=True)
+        got, info = run_gemm(cfg, a, b, kind)
+        direct += int(kind == _native.KIND_MFMA and info["lds_bytes"] == 0)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        bad = int((got.astype(np.float64) != want).sum()) + int(np.isnan(got).sum())
+        assert bad == 0, f"random edge config {i} ({info['kernel_name']}): {bad} wrong elements"
+    assert direct >= 20
 
 
 def test_random_config_sample_is_bit_exact(oracle):
