@@ -155,6 +155,41 @@ def cpu_baseline(a, b, ijk_seconds=8.0):
     }, full, M
 
 
+def power_and_clocks(kernel, A, B, C, seconds=2.0):
+    """Socket power and the clock of each XCD while `kernel` runs back to back, read once with amd-smi about a
+    second into the run.  Returns None when the tool is missing or says nothing useful (the figures are
+    evidence for the roofline discussion, not part of the measurement)."""
+    import subprocess
+    import threading
+    import torch
+    stop = threading.Event()
+
+    def spin():
+        while not stop.is_set():
+            for _ in range(100):
+                kernel.run(A, B, C)
+            torch.cuda.synchronize()
+
+    t = threading.Thread(target=spin)
+    t.start()
+    out = None
+    try:
+        time.sleep(seconds / 2)
+        p = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--json"], capture_output=True, text=True, timeout=30)
+        doc = json.loads(p.stdout)
+        gpu = (doc.get("gpu_data") if isinstance(doc, dict) else doc)[0]
+        clocks = [gpu["clock"][f"gfx_{i}"]["clk"]["value"] for i in range(8) if f"gfx_{i}" in gpu["clock"]]
+        out = {"socket_power_w": gpu["power"]["socket_power"]["value"], "gfx_clk_mhz_by_xcd": clocks,
+               "max_clk_mhz": gpu["clock"]["gfx_0"]["max_clk"]["value"], "source": "amd-smi metric --power --clock"}
+        time.sleep(seconds / 2)
+    except Exception:   # noqa: BLE001 - an absent or differently shaped tool output must not fail the benchmark
+        out = None
+    finally:
+        stop.set()
+        t.join()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -240,6 +275,14 @@ def main():
                        "roofline": {"bound": "mfma", "achieved": ach16, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
                                     "frac": ach16 / PEAK_TFLOPS["f16"], "traffic": measured_traffic(info16["kernel_name"]),
                                     "launch_ms": ms_launch16}}
+
+        if not args.no_cpu:     # (skipped in profiling runs, like the CPU leg)
+            pc = power_and_clocks(kernel16, A16, B16, C16)
+            if pc:
+                out["fp16"]["power_and_clocks"] = pc
+            pc = power_and_clocks(kernel, A, B, C)
+            if pc:
+                out["roofline"]["power_and_clocks"] = pc
 
         # the same config with bfloat16 inputs (same kernel template, same data distribution)
         cfgb = dict(cfg16)
