@@ -262,8 +262,15 @@ bool write_file_atomic(const std::string& p, const char* data, size_t n) {
 }
 
 const std::vector<std::string>& compile_flags() {
+  // -amdgpu-spill-vgpr-to-agpr=0: under register pressure the compiler parks vector registers in unused
+  // accumulation registers before it resorts to scratch memory.  Scalar-kernel configs with large thread
+  // tiles and edge predicates built that way have returned wrong values (one staging or fragment register
+  // holding another's contents) and are right with the option, at any load width and with or without
+  // branches around the edge loads; kernels that do not spill are unaffected by it.  It also makes every
+  // spill visible as scratch memory, which is what the direct-staging kernel's spill check looks at.
   static const std::vector<std::string> flags = {
       "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+      "-mllvm", "-amdgpu-spill-vgpr-to-agpr=0",
   };
   return flags;
 }

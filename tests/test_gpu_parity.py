@@ -109,7 +109,8 @@ EXACT_CASES = [
     ("f32-direct-mf16-ktail", MFMA, dict(M=252, N=248, K=560, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=0,
                                          shared_prefetch=1, reg_prefetch=1)),
     # scalar kernel, edge tiles under register pressure (16-wide thread tiles, a one-wave block with 192
-    # staging registers): shapes that returned wrong values while edge loads ran under a branch
+    # staging registers): shapes that returned wrong values when the compiler was allowed to park vector
+    # registers in accumulation registers
     ("simt-edge-16x8-both", SIMT, dict(M=244, N=376, K=112, BM=128, BN=128, BK=16, TM=16, TN=8, is_atrans=1,
                                        shared_prefetch=1, reg_prefetch=1, block_mapping=0, reduce_c_continuous=0)),
     ("simt-edge-1wave-8x16", SIMT, dict(M=124, N=124, K=133, BM=64, BN=128, BK=64, TM=8, TN=16, is_atrans=1,
@@ -118,6 +119,10 @@ EXACT_CASES = [
     ("simt-edge-1wave-8x16-glw4", SIMT, dict(M=124, N=124, K=136, BM=64, BN=128, BK=64, TM=8, TN=16, is_atrans=1,
                                              shared_prefetch=1, reg_prefetch=1, block_mapping=2, load_continuous=0,
                                              scatter=2, glw=4)),
+    ("simt-edge-16x8-unaligned", SIMT, dict(M=127, N=509, K=33, BM=128, BN=256, BK=16, TM=16, TN=8, is_atrans=1,
+                                            shared_prefetch=1, block_mapping=2, reduce_c_continuous=0)),
+    ("simt-edge-16x16-lsu2", SIMT, dict(M=124, N=253, K=66, BM=128, BN=128, BK=16, TM=16, TN=16, is_atrans=1,
+                                        shared_prefetch=1, reg_prefetch=1, lsu=2, reduce_c_continuous=0)),
     # fp64 on the matrix cores (16x16x4 instructions, two k values per 16-byte chunk)
     ("mfma-f64", MFMA, dict(M=256, N=256, K=128, dtype=8, scatter=2)),
     ("mfma-f64-at0-both", MFMA, dict(M=256, N=192, K=136, dtype=8, scatter=2, is_atrans=0, shared_prefetch=1,
