@@ -216,7 +216,7 @@ int reference_lds_bytes(const MatmulConfig& c) {
 
 // (That kernel keeps 2..4 stages of (BM+BN)*BK*2 bytes in static LDS: as many as fit in 160 KiB.)
 // Must state the same rule as DirectPlan<C>::ELIGIBLE in kcg_device_direct.h (a static_assert there
-// compares the two): 16-bit inputs or fp32 throughout, a K remainder of whole k-steps, both prefetch flags, LOAD_CONTINUOUS, 128-bit load
+// compares the two): 16-bit inputs or fp32 throughout, at least one full K tile, both prefetch flags, LOAD_CONTINUOUS, 128-bit load
 // widths, power-of-two tiles that split evenly into 1 KiB wave fetches, at least two rows of
 // matrix-core tiles per wave, and two LDS stages within 160 KiB.
 bool mfma_direct(const MatmulConfig& c) {
@@ -231,8 +231,8 @@ bool mfma_direct(const MatmulConfig& c) {
   const int mf = es == 2 ? ((c.BK % 32 == 0 || !fits32) ? 16 : 32) : (fits32 ? 32 : 16);
   const int ks = g * (64 / mf);
   if (c.BK % ks) return false;
-  // edge tiles in M and N are handled; K needs one full tile and a remainder of whole k-steps
-  if (c.K < c.BK || (c.K % c.BK) % ks) return false;
+  // edge tiles in M and N are handled; K needs one full tile (a remainder is a multiple of g like K itself)
+  if (c.K < c.BK) return false;
   if (p.WM / mf < 2) return false;                       // the K loop streams A fragments row by row
   const int nw = c.BLM * c.BLN;
   if (!is_pow2(c.BM) || !is_pow2(c.BN) || !is_pow2(c.BK) || c.BM < 64 || c.BN < 64) return false;

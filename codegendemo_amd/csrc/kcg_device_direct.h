@@ -22,7 +22,8 @@ namespace kcg {
 // Edge tiles cost the K loop nothing: a lane whose chunk lies outside the matrix (rows or columns
 // beyond M or N; k beyond K in the last, partial K tile) fetches a chunk of the same tile that does exist
 // instead.  What lands in LDS for it only ever reaches accumulators of rows/columns that are not stored
-// (M, N) or is not read at all (the partial K tile computes only the k-steps it has).
+// (M, N) or is not read at all (the partial K tile computes only the k-steps it has; where its last
+// k-step is itself partial, the lanes that hold k values beyond K clear their fragments before use).
 // The bank swizzle is applied on the fetch side: the lane that fills physical chunk c' of a row fetches
 // logical chunk c' ^ swz(row), and readers look chunk c up at c ^ swz(row).
 // =============================================================================================
@@ -85,8 +86,8 @@ struct DirectPlan {
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
-      // edge tiles in M and N are fine; K needs one full tile and a remainder of whole k-steps
-      SPW > 0 && C::K >= C::BK && (C::K % C::BK) % KS == 0 && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
+      // edge tiles in M and N are fine; K needs one full tile (its remainder is a multiple of G like K itself)
+      SPW > 0 && C::K >= C::BK && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
       (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
       (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
@@ -121,7 +122,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int KH = 64 / MF, KS = P::KS, SPW = P::SPW;
   constexpr int TMI = WM / MF, TNI = WN / MF, NM = P::NM, NW = P::NW;
   constexpr int KT = K / BK;                            // full K tiles
-  constexpr int KR = K % BK, SPWT = KR / KS;            // the remainder: one more tile of SPWT k-steps
+  constexpr int KR = K % BK, SPWT = cdiv(KR, KS);       // the remainder: one more tile of SPWT k-steps (the last may be partial)
   constexpr int KTT = KT + (KR > 0 ? 1 : 0);
   constexpr bool EDGE_M = M % BM != 0, EDGE_N = N % BN != 0;
   constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
@@ -255,6 +256,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragTr {                                    // 16-bit, row-contiguous tile: two transposing 64-bit reads
     u32x2 h[2];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
+    __device__ __forceinline__ void keep_if(bool keep) { h[0] = keep ? h[0] : u32x2{0, 0}; h[1] = keep ? h[1] : u32x2{0, 0}; }
     __device__ __forceinline__ Frag get() const {
       const u32x4 v = {h[0].x, h[0].y, h[1].x, h[1].y};
       return __builtin_bit_cast(Frag, v);
@@ -263,6 +265,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragS4 {                                    // 32-bit, row-contiguous tile: four 32-bit reads
     unsigned w[4];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3])); }
+    __device__ __forceinline__ void keep_if(bool keep) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = keep ? w[e] : 0u;
+    }
     __device__ __forceinline__ Frag get() const {
       const u32x4 v = {w[0], w[1], w[2], w[3]};
       return __builtin_bit_cast(Frag, v);
@@ -271,6 +277,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragLd {                                    // k-contiguous tile: one 128-bit read
     u32x4 q;
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(q)); }
+    __device__ __forceinline__ void keep_if(bool keep) { q = keep ? q : u32x4{0, 0, 0, 0}; }
     __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
   };
   typedef typename Select<ES == 2, FragTr, FragS4>::type FragRc;
@@ -437,9 +444,15 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     constexpr bool HP = decltype(hasp)::value && SPREAD > TAIL;
     const TileBase tbn = tile_base(HN ? kt + NST : 0);
     const TileBase tbp = tile_base(HP ? kt - 1 + NST : 0);
+    // In the partial K tile a k-step may reach beyond K: every fragment layout of this kernel gives a lane
+    // the G consecutive k values that start at S*KS + G*(lane/MF), so such a lane holds nothing but
+    // k >= K (what was fetched in their place is arbitrary) and clears its fragments.
+    constexpr bool PARTIAL = KR > 0 && NS == SPWT && decltype(has1)::value == false && (KR % KS != 0);
     static_for<0, NS>([&](auto s_c) {
       constexpr int S = decltype(s_c)::value;
       constexpr bool LAST = (S == NS - 1);
+      constexpr bool MASK = PARTIAL && LAST;
+      const bool keep = S * KS + G * fgrp < KR;
       constexpr int PB = (CUR * SPW + S) & 1;       // half of the B double buffer this step computes from
       constexpr bool NEXT = !LAST || H1;            // a next step exists, its fragments are read under this one
       static_for<0, TMI>([&](auto i_c) {
@@ -467,6 +480,20 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         if constexpr (I == 0) {
 #pragma unroll
           for (int j = 0; j < TNI; ++j) fb[PB][j].pin();
+        }
+        if constexpr (MASK) {
+          // (pinned again behind the selects: they must have been issued before the wait state that
+          // separates them from the matrix-core instruction reading their results)
+          fa[I].keep_if(keep);
+          fa[I].pin();
+          if constexpr (I == 0) {
+#pragma unroll
+            for (int j = 0; j < TNI; ++j) {
+              fb[PB][j].keep_if(keep);
+              fb[PB][j].pin();
+            }
+          }
+          asm volatile("s_nop 1" ::: "memory");
         }
         if constexpr (I + DA < TMI) load_a(IntC<CUR>(), IntC<S>(), IntC<I + DA>(), &fa[I + DA]);
         else if constexpr (!LAST) load_a(IntC<CUR>(), IntC<S + 1>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);

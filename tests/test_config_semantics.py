@@ -171,19 +171,20 @@ def test_instantiation_source_carries_the_config():
 
 @pytest.mark.parametrize("shape,kw,direct", [
     ((4096, 1536, 1000), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # K = 62*16 + 8: one k-step of 8 left over
-    ((4096, 1536, 1004), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),     # remainder 12 is not a whole k-step
+    ((4096, 1536, 1004), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # remainder 12: a whole k-step and half of one
+    ((4096, 1536, 1002), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),     # K is not a multiple of the 16-byte vector
     ((4096, 1536, 8), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),        # not even one full K tile
     ((200, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),         # rows and columns beyond M and N
     ((202, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),        # M is not a multiple of the 16-byte vector
     ((256, 256, 992), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),    # 16x16x32 tiles: k-steps of 32
-    ((256, 256, 1008), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), False),  # remainder 48
+    ((256, 256, 1008), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # remainder 48 = 1.5 k-steps
+    ((256, 256, 1004), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), False),  # K % 8 != 0
     ((256, 256, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4, load_continuous=0), False),
     ((256, 256, 1024), dict(BM=128, BN=128, BK=16, TM=8, TN=8, dtype=8, scatter=2), False),  # fp64: register staging only
 ])
 def test_direct_staging_eligibility(shape, kw, direct):
     """Which matrix-core configs get the direct global->LDS kernel: both prefetch flags, LOAD_CONTINUOUS and
-    128-bit loads; any M and N that are multiples of the 16-byte vector; K at least one tile with a remainder
-    of whole k-steps.  (The device template re-derives the rule and a static_assert compares the two.)"""
+    128-bit loads; any M, N and K that are multiples of the 16-byte vector, K at least one tile.  (The device template re-derives the rule and a static_assert compares the two.)"""
     full = dict(is_atrans=0, shared_prefetch=1, reg_prefetch=1)
     full.update(kw)
     src = _native.instantiation_source(vals(make_config(*shape, **full)), _native.KIND_MFMA)

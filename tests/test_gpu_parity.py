@@ -106,6 +106,13 @@ EXACT_CASES = [
                                           shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-edge-256", MFMA, dict(M=260, N=516, K=1064, BM=256, BN=256, TM=16, TN=16, BK=32, is_atrans=0,
                                        shared_prefetch=1, reg_prefetch=1)),
+    # K remainders that end inside a k-step: the lanes holding k >= K clear their fragments
+    ("f32-direct-kpart", MFMA, dict(M=256, N=256, K=1004, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=0,
+                                    shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-kpart-bk32-at1", MFMA, dict(M=200, N=136, K=1020, BM=128, BN=128, TM=8, TN=8, BK=32, is_atrans=1,
+                                             shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-mf16-kpart-at1", MFMA, dict(M=252, N=248, K=572, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=1,
+                                             shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-mf16-ktail", MFMA, dict(M=252, N=248, K=560, BM=128, BN=64, TM=8, TN=2, BK=32, is_atrans=0,
                                          shared_prefetch=1, reg_prefetch=1)),
     # scalar kernel, edge tiles under register pressure (16-wide thread tiles, a one-wave block with 192
@@ -197,6 +204,12 @@ HALF_CASES = [
     # edge tiles through the direct-staging kernel: partial last K tile, rows/columns beyond M and N
     ("f16-direct-ktail", dict(M=256, N=256, K=992, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
                               shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-kpart", dict(M=256, N=256, K=1000, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
+                              shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-direct-kpart-at1", dict(M=200, N=136, K=72, dtype=3, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8, BK=64,
+                                   shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-kpart-mf32", dict(M=256, N=256, K=408, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=16,
+                                   shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-edge-at1", dict(M=200, N=136, K=160, dtype=2, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8,
                                  BK=64, shared_prefetch=1, reg_prefetch=1)),
     ("bf16-direct-256-edge", dict(M=264, N=520, K=1120, dtype=3, dtype_c=4, is_atrans=0, BM=256, BN=256, TM=16, TN=16,

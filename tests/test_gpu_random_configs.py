@@ -100,7 +100,7 @@ def random_edge_configs(n_matrix=50, n_simt=30, n_direct=25, seed=20250311):
                 have[kind] += 1
         except (ValueError, _native.KcgError):
             continue
-    # ... and configs that take the direct-staging kernel with such shapes (K remainders of whole k-steps)
+    # ... and configs that take the direct-staging kernel with such shapes (K remainders included)
     n = 0
     while n < n_direct:
         dtype = rng.choice([2, 3, 4, 4])
