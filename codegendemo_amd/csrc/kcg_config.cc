@@ -226,8 +226,8 @@ bool mfma_direct(const MatmulConfig& c) {
   const int g = 16 / es;                                  // elements per 16-byte chunk
   if (!c.SHMP || !c.REGP || !c.LC || c.LSU != 1 || c.GLW_A != g || c.GLW_B != g) return false;
   // this path picks its own matrix-core tile: for 16-bit inputs 16x16x32 whenever the K tile is a
-  // multiple of 32; for fp32 the larger tile where the wave tile allows
-  const bool fits32 = p.WM % 32 == 0 && p.WN % 32 == 0;
+  // multiple of 32; for fp32 the larger tile where the wave tile holds two rows of them
+  const bool fits32 = p.WM % 32 == 0 && p.WN % 32 == 0 && p.WM / 32 >= 2;   // two rows of tiles per wave
   const int mf = es == 2 ? ((c.BK % 32 == 0 || !fits32) ? 16 : 32) : (fits32 ? 32 : 16);
   const int ks = g * (64 / mf);
   if (c.BK % ks) return false;

@@ -74,7 +74,8 @@ struct DirectPlan {
 #define KCG_DIRECT_MF 0               /* 16 or 32 forces the matrix-core tile of the direct-staging kernel */
 #endif
   static constexpr int G = 16 / ES;                               // elements per 16-byte chunk
-  static constexpr bool FITS32 = WM % 32 == 0 && WN % 32 == 0;
+  // (the streaming K loop wants two rows of matrix-core tiles per wave: a 32-row wave tile takes 16x16 tiles)
+  static constexpr bool FITS32 = WM % 32 == 0 && WN % 32 == 0 && WM / 32 >= 2;
   static constexpr int MF = KCG_DIRECT_MF ? KCG_DIRECT_MF
                             : ES == 2 ? ((C::BK % 32 == 0 || !FITS32) ? 16 : 32)
                                       : (FITS32 ? 32 : 16);       // fp32: no such difference, the larger tile reads less
