@@ -235,7 +235,7 @@ bool mfma_direct(const MatmulConfig& c) {
   if (c.K < c.BK) return false;
   if (p.WM / mf < 2) return false;                       // the K loop streams A fragments row by row
   const int nw = c.BLM * c.BLN;
-  if (!is_pow2(c.BM) || !is_pow2(c.BN) || !is_pow2(c.BK) || c.BM < 64 || c.BN < 64) return false;
+  if (!is_pow2(c.BM) || !is_pow2(c.BN) || !is_pow2(c.BK) || c.BM < 32 || c.BN < 32) return false;
   if ((c.BM * c.BK / g) % (64 * nw) || (c.BN * c.BK / g) % (64 * nw)) return false;
   if (c.M % g || c.N % g || c.K % g) return false;
   const long lim = 1L << 31;                              // 32-bit byte offsets per lane inside a tile panel

@@ -88,7 +88,7 @@ struct DirectPlan {
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
       // edge tiles in M and N are fine; K needs one full tile (its remainder is a multiple of G like K itself)
-      SPW > 0 && C::K >= C::BK && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 64 && C::BN >= 64 &&
+      SPW > 0 && C::K >= C::BK && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 32 && C::BN >= 32 &&
       (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
       (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane

@@ -180,6 +180,8 @@ def test_instantiation_source_carries_the_config():
     ((256, 256, 1008), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # remainder 48 = 1.5 k-steps
     ((256, 256, 1004), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), False),  # K % 8 != 0
     ((256, 256, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4, load_continuous=0), False),
+    ((1024, 1024, 1024), dict(BM=32, BN=32, BK=16, TM=4, TN=4, is_atrans=1), True),        # one wave, 2x2 tiles of 16x16
+    ((1024, 1024, 1024), dict(BM=32, BN=64, BK=16, TM=2, TN=8, warp_layout=(8, 8)), False),  # 16-row wave tile: one row of tiles
     ((256, 256, 1024), dict(BM=128, BN=128, BK=16, TM=8, TN=8, dtype=8, scatter=2), False),  # fp64: register staging only
 ])
 def test_direct_staging_eligibility(shape, kw, direct):

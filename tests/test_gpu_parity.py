@@ -106,6 +106,13 @@ EXACT_CASES = [
                                           shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-edge-256", MFMA, dict(M=260, N=516, K=1064, BM=256, BN=256, TM=16, TN=16, BK=32, is_atrans=0,
                                        shared_prefetch=1, reg_prefetch=1)),
+    # 32-wide block tiles (one wave of 32x32, two of 32x32 side by side): 8 chunks per tile row
+    ("f32-direct-32x32-1wave", MFMA, dict(M=96, N=160, K=272, BM=32, BN=32, TM=4, TN=4, BK=16, is_atrans=1,
+                                          shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-32x64-edge", MFMA, dict(M=100, N=136, K=108, BM=32, BN=64, TM=4, TN=4, BK=32, is_atrans=0,
+                                         shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-64x32-at1", MFMA, dict(M=128, N=96, K=520, BM=64, BN=32, TM=8, TN=4, BK=8, is_atrans=1,
+                                        shared_prefetch=1, reg_prefetch=1)),
     # K remainders that end inside a k-step: the lanes holding k >= K clear their fragments
     ("f32-direct-kpart", MFMA, dict(M=256, N=256, K=1004, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=0,
                                     shared_prefetch=1, reg_prefetch=1)),
@@ -204,6 +211,10 @@ HALF_CASES = [
     # edge tiles through the direct-staging kernel: partial last K tile, rows/columns beyond M and N
     ("f16-direct-ktail", dict(M=256, N=256, K=992, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
                               shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-32x32-1wave-at1", dict(M=96, N=160, K=288, dtype=2, dtype_c=4, is_atrans=1, BM=32, BN=32, TM=4, TN=4,
+                                        BK=32, shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-direct-32x64-edge", dict(M=104, N=136, K=200, dtype=3, dtype_c=4, is_atrans=0, BM=32, BN=64, TM=4, TN=4,
+                                    BK=64, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-kpart", dict(M=256, N=256, K=1000, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=64,
                               shared_prefetch=1, reg_prefetch=1)),
     ("bf16-direct-kpart-at1", dict(M=200, N=136, K=72, dtype=3, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8, BK=64,
