@@ -102,7 +102,21 @@ struct DirectPlan {
   static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
   static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
   static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
-  static constexpr int NST_CAP = NST_MAX < 2 ? 2 : (NST_MAX > 4 ? 4 : NST_MAX);
+  // Two blocks on a compute unit beat one block with deeper staging when the launch has more blocks than the
+  // chip has compute units (256): one block's prologue, barrier waits and C stores run under the other's
+  // matrix work (measured 2-5 % at 4096x1536x1000, 2048^3 and 4096^3 with 128x64 and 128x128 tiles).  Where
+  // two blocks fit the register file (512 registers per lane and SIMD, a block's waves dealt evenly over
+  // the four SIMDs: a wave holds WM*WN/64 accumulators and some 64 registers of fragments and addresses) the
+  // stages are limited to half of the LDS.
+#ifndef KCG_DIRECT_NST
+#define KCG_DIRECT_NST 0              /* upper limit of the number of LDS stages; 0: the rule below */
+#endif
+  static constexpr int GRID_BLOCKS = ((C::M + C::BM - 1) / C::BM) * ((C::N + C::BN - 1) / C::BN);
+  static constexpr bool PAIR = GRID_BLOCKS > 256 && NW % 4 == 0 && (WM * WN / 64 + 64) * (NW / 2) <= 512 &&
+                               2 * STAGE_BYTES <= 80 * 1024;
+  static constexpr int NST_LIMIT = KCG_DIRECT_NST > 0 ? KCG_DIRECT_NST : (PAIR ? (80 * 1024) / STAGE_BYTES : 4);
+  static constexpr int NST_TOP = NST_LIMIT > 4 ? 4 : NST_LIMIT;
+  static constexpr int NST_CAP = NST_MAX < 2 ? 2 : (NST_MAX > NST_TOP ? NST_TOP : NST_MAX);
   static constexpr int NST = (SPW % 2 == 1 && NST_CAP % 2 == 1) ? NST_CAP - 1 : NST_CAP;
   // the host picks the path (it must size dynamic LDS accordingly): both sides have to agree on the
   // rule; the host may still decline an eligible config (a direct-staging build that would spill)
