@@ -93,7 +93,8 @@ struct DirectPlan {
       (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
       (long)C::BM * C::K * ES < (1L << 31) && (long)C::BK * C::M * ES < (1L << 31) && (long)C::BK * C::N * ES < (1L << 31);
-  // LDS stages: as many as fit in 160 KiB, at most 4 (fetch distance = NST-1 K tiles); an even number
+  // LDS stages: as many as fit in 160 KiB (or in half of it, see PAIR below), at most 4 (fetch distance =
+  // NST-1 K tiles); an even number
   // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
   static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * ES;
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;

@@ -373,3 +373,46 @@ def test_tuned_4096_kernels_are_bit_exact_on_integers(oracle, which):
     assert not np.isnan(got).any()
     bad = np.argwhere(got != want)
     assert bad.size == 0, f"tuned {which}: {len(bad)} mismatches, first at {bad[:5].tolist()}"
+
+
+def test_config3_fp32_4096_uniform(oracle):
+    """BASELINE config 3: fp32 4096^3, row-major A[M,K], uniform[-1,1), the tuned kernel bench.py launches:
+    a 64-row panel in full against the oracle, plus the column-sum identity over the whole output."""
+    cfg = dict(_tuned("gemm_4096_fp32.json"))
+    M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+    a = SI.uniform((M, K), SI.STREAM_A)
+    b = SI.uniform((K, N), SI.STREAM_B)
+    rows = (3000, 3064)
+    want = oracle.matmul(a, b, a_trans=False, rows=rows)
+    tol = fp32_tolerance(K, a, b)
+    print("[case] config3 tuned fp32 4096^3", flush=True)
+    got, _ = run_gemm(cfg, a, b)
+    assert not np.isnan(got).any()
+    err = float(np.abs(got[rows[0]:rows[1]] - want).max())
+    print(f"        panel max|err|={err:.3e} tol={tol:.3e}", flush=True)
+    assert err <= tol
+    assert err <= 1e-3                       # far inside the contract
+    lhs = got.astype(np.float64).sum(axis=0)
+    rhs = a.astype(np.float64).sum(axis=0) @ b.astype(np.float64)
+    assert np.abs(lhs - rhs).max() <= tol * np.sqrt(M)
+
+
+@pytest.mark.parametrize("index", range(5))
+def test_tuned_edge_shape_kernels_are_bit_exact_on_integers(oracle, index):
+    """The five best configs of the 4096 x 1536 x 1000 sweep (768 or more blocks, two of them resident per
+    compute unit, a partial last K tile): integers in [-2, 2] give sums that are exact in fp32, so the whole
+    result must equal the oracle bit for bit."""
+    import json
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "codegendemo_amd", "TunedConfigs", "gemm_4096x1536x1000_fp32.json")) as f:
+        cfg = json.load(f)["cfgs"][index]
+    M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+    a = SI.small_ints((M, K), SI.STREAM_A, lim=2)
+    b = SI.small_ints((K, N), SI.STREAM_B, lim=2)
+    print(f"[case] tuned edge shape #{index} {M}x{N}x{K}", flush=True)
+    got, _ = run_gemm(cfg, a, b)
+    want = oracle.matmul(a, b, a_trans=False)
+    assert not np.isnan(got).any()
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, f"tuned edge config {index}: {len(bad)} mismatches, first at {bad[:5].tolist()}"
