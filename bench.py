@@ -36,6 +36,7 @@ MEASURED_TRAFFIC_BYTES = {
     "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x8_BTmnk256x256x32_BLmn2x4": (2 * 196730 + 65569) * 1024,
     "DTabcfloat32xfloat32xfloat32_AT0_TTmn16x16_BTmnk256x256x32_BLmn2x2": (2 * 196749 + 65536) * 1024,
     "DTabcfloat16xfloat16xfloat32_AT0_TTmn16x16_BTmnk256x256x64_BLmn2x2": (2 * 98428 + 65536) * 1024,
+    "MNK4096x1536x1000_DTabcfloat32xfloat32xfloat32_AT0_TTmn4x8_BTmnk64x128x32_BLmn2x2": (2 * 43119 + 24576) * 1024,
 }
 
 
@@ -251,7 +252,10 @@ def main():
         "value": value, "unit": "TFLOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "fp32 GEMM M=N=K=4096, row-major A[M,K] B[K,N], uniform[-1,1) seeded, tuned config",
+        "config": {"workload": ("fp32 GEMM M=N=K=4096" if (kpm.M, kpm.N, kpm.K) == (4096, 4096, 4096)
+                                else f"fp32 GEMM M={kpm.M} N={kpm.N} K={kpm.K} (--fp32-config)")
+                               + (", A stored [K,M]" if kpm.isATranspose else ", row-major A[M,K]")
+                               + " B[K,N], uniform[-1,1) seeded, tuned config",
                    "kernel": info["kernel_name"], "kind": {1: "simt", 2: "mfma"}[info["kind"]],
                    "lds_bytes": info["lds_bytes"], "grid": info["grid"][0], "block": info["block"][0]},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS["f32"], "unit": "TFLOP/s",
