@@ -83,6 +83,15 @@ def make_inputs(kpm, dist):
     return a, b, A, B, C
 
 
+def make_inputs_host(kpm16):
+    """The fp16 workload's operands as the kernel sees them: normal(0, 0.5) rounded to fp16, upcast to fp32."""
+    import numpy as np
+    from codegendemo_amd.kcg import SeededInputs as SI
+    a = SI.normal((kpm16.M, kpm16.K), SI.STREAM_A, std=0.5).astype(np.float16).astype(np.float32)
+    b = SI.normal((kpm16.K, kpm16.N), SI.STREAM_B, std=0.5).astype(np.float16).astype(np.float32)
+    return a, b
+
+
 def time_steps(kernel, A, B, C, steps, warmup):
     """-> (wall ms per step over K steps, HIP-event average launch duration in ms)."""
     import torch
@@ -282,6 +291,20 @@ def main():
                                     "launch_ms": ms_launch16}}
 
         if not args.no_cpu:     # (skipped in profiling runs, like the CPU leg)
+            # parity of the fp16 result: a 64-row panel against the oracle run on the upcast fp16 values;
+            # bar: 2e-2 relative to the RMS magnitude of C
+            from tests import oracle_binding
+            a16h, b16h = make_inputs_host(kpm16)
+            r0, r1 = 2048, 2112
+            want16 = oracle_binding.load().matmul(a16h, b16h, 0, rows=(r0, r1))
+            got16 = C16[r0:r1].cpu().numpy()
+            scale16 = float(np.sqrt(np.mean(want16.astype(np.float64) ** 2)))
+            rel16 = float(np.abs(got16 - want16).max()) / scale16
+            out["fp16"]["parity"] = {"rows_checked": r1 - r0, "max_rel_err": rel16, "tolerance": 2e-2, "ok": bool(rel16 <= 2e-2)}
+            if not rel16 <= 2e-2:
+                print(json.dumps(out))
+                print("bench.py: fp16 GPU result differs from the oracle beyond tolerance", file=sys.stderr)
+                sys.exit(1)
             pc = power_and_clocks(kernel16, A16, B16, C16)
             if pc:
                 out["fp16"]["power_and_clocks"] = pc

@@ -334,8 +334,9 @@ def test_config5_fp16_4096(oracle):
     rows = (1024, 1088)
     want = oracle.matmul(a, b, a_trans=False, rows=rows)
     scale = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
-    for kw in CONFIG5_KERNELS:
-        cfg = make_config(M, N, K, dtype=2, dtype_c=4, is_atrans=0, **kw)
+    cfgs = [("tuned", dict(_tuned("gemm_4096_fp16.json")))]        # the kernel bench.py launches
+    cfgs += [(str(kw), make_config(M, N, K, dtype=2, dtype_c=4, is_atrans=0, **kw)) for kw in CONFIG5_KERNELS]
+    for kw, cfg in cfgs:
         print(f"[case] config5 {kw}", flush=True)
         got, _ = run_gemm(cfg, a, b, MFMA)
         assert not np.isnan(got).any()
