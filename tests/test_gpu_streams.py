@@ -37,3 +37,42 @@ def test_launch_is_ordered_on_a_side_stream(oracle):
     got = c_dev.cpu().numpy()
     kernel.unload()
     assert np.array_equal(got, 2.0 * want)
+
+
+def test_launch_can_be_captured_in_a_hip_graph(oracle):
+    """A launch through the boundary allocates nothing and synchronises nothing, so a caller may capture it
+    into a HIP graph (once the module is loaded: the first run of a kernel loads it, which is not capturable).
+    The graph is replayed four times on different operands with eager work and synchronisations in between;
+    every replay must equal the eager result and the oracle bit for bit (small integers)."""
+    import torch
+    kpm, ui, kernel, info = build_kernel(CONFIG)
+    b = SI.small_ints((K, N), SI.STREAM_B)
+    b_dev = to_device(b, torch.float32)
+    a_dev = torch.zeros((M, K), dtype=torch.float32, device="cuda:0")
+    c_dev = torch.zeros((M, N), dtype=torch.float32, device="cuda:0")
+    c_eager = torch.zeros((M, N), dtype=torch.float32, device="cuda:0")
+    print("[case] graph capture 512^3", flush=True)
+    kernel.run(a_dev, b_dev, c_dev)      # loads the module
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()           # default priority
+    with torch.cuda.graph(graph, stream=side):
+        kernel.run(a_dev, b_dev, c_dev)
+        c_dev.mul_(2.0)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        a = SI.small_ints((M, K), SI.STREAM_A, seed=SI.SEED + rep)
+        a_dev.copy_(to_device(a, torch.float32))
+        c_dev.fill_(float("nan"))        # a fill kernel, eager, outside the graph
+        torch.cuda.synchronize()
+        print(f"        replay {rep}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        kernel.run(a_dev, b_dev, c_eager)
+        c_eager.mul_(2.0)
+        torch.cuda.synchronize()
+        got = c_dev.cpu().numpy()
+        assert np.array_equal(got, c_eager.cpu().numpy()), f"replay {rep} differs from the eager result"
+        assert np.array_equal(got, 2.0 * oracle.matmul(a, b, a_trans=False)), f"replay {rep} differs from the oracle"
+    del graph
+    kernel.unload()
