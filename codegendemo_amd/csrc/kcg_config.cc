@@ -217,7 +217,7 @@ int reference_lds_bytes(const MatmulConfig& c) {
 // (That kernel keeps 2..4 stages of (BM+BN)*BK*2 bytes in static LDS: as many as fit in 160 KiB.)
 // Must state the same rule as DirectPlan<C>::ELIGIBLE in kcg_device_direct.h (a static_assert there
 // compares the two): 16-bit inputs or fp32 throughout, at least one full K tile, both prefetch flags, LOAD_CONTINUOUS, 128-bit load
-// widths, power-of-two tiles that split evenly into 1 KiB wave fetches, at least two rows of
+// widths, tiles (powers of two or multiples of 16 chunks) that split evenly into 1 KiB wave fetches, at least two rows of
 // matrix-core tiles per wave, and two LDS stages within 160 KiB.
 bool mfma_direct(const MatmulConfig& c) {
   MfmaPlan p = plan_mfma(c);
@@ -235,7 +235,9 @@ bool mfma_direct(const MatmulConfig& c) {
   if (c.K < c.BK) return false;
   if (p.WM / mf < 2) return false;                       // the K loop streams A fragments row by row
   const int nw = c.BLM * c.BLN;
-  if (!is_pow2(c.BM) || !is_pow2(c.BN) || !is_pow2(c.BK) || c.BM < 32 || c.BN < 32) return false;
+  // tile extents: a power of two or a multiple of 16 chunks (the bank swizzle works on aligned groups of 16 chunks)
+  auto tile_ok = [g](int x) { return is_pow2(x) || (x > 0 && x % (16 * g) == 0); };
+  if (!tile_ok(c.BM) || !tile_ok(c.BN) || !is_pow2(c.BK) || c.BM < 32 || c.BN < 32) return false;
   if ((c.BM * c.BK / g) % (64 * nw) || (c.BN * c.BK / g) % (64 * nw)) return false;
   if (c.M % g || c.N % g || c.K % g) return false;
   const long lim = 1L << 31;                              // 32-bit byte offsets per lane inside a tile panel

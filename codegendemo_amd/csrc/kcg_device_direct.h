@@ -84,11 +84,14 @@ struct DirectPlan {
   static constexpr int NM = (WM / MF) * (WN / MF);
   static constexpr int SPW = (C::BK % KS == 0) ? C::BK / KS : 0;
   static constexpr bool pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+  // block tile extents: a power of two, or a multiple of 16 chunks (the bank swizzle of a row-contiguous
+  // tile exchanges chunks inside aligned groups of 16, so a row must consist of whole groups): 192, 320, ...
+  static constexpr bool tile_ok(int x) { return pow2(x) || (x > 0 && x % (16 * G) == 0); }
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
       // edge tiles in M and N are fine; K needs one full tile (its remainder is a multiple of G like K itself)
-      SPW > 0 && C::K >= C::BK && WM / MF >= 2 && pow2(C::BM) && pow2(C::BN) && pow2(C::BK) && C::BM >= 32 && C::BN >= 32 &&
+      SPW > 0 && C::K >= C::BK && WM / MF >= 2 && tile_ok(C::BM) && tile_ok(C::BN) && pow2(C::BK) && C::BM >= 32 && C::BN >= 32 &&
       (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
       (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
@@ -175,9 +178,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // 32-bit: a fragment read is four 32-bit reads; in each, MF lanes read consecutive columns of one row
   // and the 64/MF lane groups read rows 4 apart, which must fall into different bank ranges.
   auto swz_n = [](int k, int nch) {
-    if constexpr (ES == 2) return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & (nch - 1);
-    else if constexpr (MF == 32) return (((k >> 2) & 1) << 3) & (nch - 1);
-    else return (((k >> 2) & 3) << 2) & (nch - 1);
+    const int mask = nch >= 16 ? 15 : nch - 1;          // nch: a power of two below 16, or a multiple of 16
+    if constexpr (ES == 2) return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & mask;
+    else if constexpr (MF == 32) return (((k >> 2) & 1) << 3) & mask;
+    else return (((k >> 2) & 3) << 2) & mask;
   };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------

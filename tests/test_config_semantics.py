@@ -183,6 +183,11 @@ def test_instantiation_source_carries_the_config():
     ((1024, 1024, 1024), dict(BM=32, BN=32, BK=16, TM=4, TN=4, is_atrans=1), True),        # one wave, 2x2 tiles of 16x16
     ((1024, 1024, 1024), dict(BM=32, BN=64, BK=16, TM=2, TN=8, warp_layout=(8, 8)), False),  # 16-row wave tile: one row of tiles
     ((256, 256, 1024), dict(BM=128, BN=128, BK=16, TM=8, TN=8, dtype=8, scatter=2), False),  # fp64: register staging only
+    # tile extents that are not powers of two: whole groups of 16 chunks (64 fp32 / 128 16-bit elements) per row
+    ((4096, 1536, 1000), dict(BM=64, BN=192, BK=32, TM=4, TN=12), True),
+    ((4096, 1536, 1000), dict(BM=128, BN=96, BK=32, TM=8, TN=6, scatter=2), False),          # 24 chunks per row
+    ((768, 768, 512), dict(BM=128, BN=384, BK=32, TM=8, TN=12, dtype=2, dtype_c=4), True),
+    ((768, 768, 512), dict(BM=128, BN=192, BK=32, TM=8, TN=12, dtype=2, dtype_c=4), False),  # 24 chunks per row
 ])
 def test_direct_staging_eligibility(shape, kw, direct):
     """Which matrix-core configs get the direct global->LDS kernel: both prefetch flags, LOAD_CONTINUOUS and

@@ -113,6 +113,16 @@ EXACT_CASES = [
                                          shared_prefetch=1, reg_prefetch=1)),
     ("f32-direct-64x32-at1", MFMA, dict(M=128, N=96, K=520, BM=64, BN=32, TM=8, TN=4, BK=8, is_atrans=1,
                                         shared_prefetch=1, reg_prefetch=1)),
+    # block tiles that are not powers of two (whole groups of 16 chunks per tile row): 192 columns, 192 rows in
+    # both A layouts, edges in M, N and K
+    ("f32-direct-64x192", MFMA, dict(M=256, N=768, K=544, BM=64, BN=192, TM=4, TN=12, BK=32, is_atrans=0,
+                                     shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-192x64-at1-edge", MFMA, dict(M=500, N=200, K=1000, BM=192, BN=64, TM=12, TN=4, BK=16, is_atrans=1,
+                                              shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-192x128-at0-edge", MFMA, dict(M=388, N=516, K=264, BM=192, BN=128, TM=12, TN=8, BK=32, is_atrans=0,
+                                               shared_prefetch=1, reg_prefetch=1)),
+    ("f32-direct-128x192-8w", MFMA, dict(M=512, N=1536, K=1000, BM=128, BN=192, TM=8, TN=6, BK=32, is_atrans=0,
+                                         scatter=2, shared_prefetch=1, reg_prefetch=1)),
     # K remainders that end inside a k-step: the lanes holding k >= K clear their fragments
     ("f32-direct-kpart", MFMA, dict(M=256, N=256, K=1004, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=0,
                                     shared_prefetch=1, reg_prefetch=1)),
@@ -165,6 +175,10 @@ HALF_CASES = [
     ("f16-out16", dict(M=256, N=256, K=128, dtype=2, is_atrans=0, BK=32)),
     ("f16-direct-at1", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=1, BM=128, BN=128, TM=8, TN=8, BK=64,
                             shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-128x384", dict(M=256, N=768, K=544, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=384, TM=8, TN=12, BK=32,
+                                shared_prefetch=1, reg_prefetch=1)),
+    ("f16-direct-384x128-at1-edge", dict(M=776, N=248, K=552, dtype=2, dtype_c=4, is_atrans=1, BM=384, BN=128, TM=12, TN=8,
+                                         BK=32, shared_prefetch=1, reg_prefetch=1)),
     ("f16-direct-bk32", dict(M=256, N=384, K=224, dtype=2, dtype_c=4, is_atrans=0, BM=128, BN=128, TM=8, TN=8, BK=32,
                              shared_prefetch=1, reg_prefetch=1)),
     ("f16-wl4x16-shmp", dict(M=256, N=256, K=256, dtype=2, dtype_c=4, is_atrans=0, warp_layout=(4, 16), BM=64, BN=64,
