@@ -14,6 +14,7 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 CFG_LEN = 31
 KIND_AUTO, KIND_SIMT, KIND_MFMA = 0, 1, 2
 KCG_OK = 0
+EPILOGUE_NONE, EPILOGUE_ALPHA_BETA = 0, 1
 ERR_INVALID_CONFIG, ERR_COMPILE, ERR_IO, ERR_HIP, ERR_ARGUMENT = -1, -2, -3, -4, -5
 
 
@@ -49,7 +50,7 @@ EXPORTS = (
     "kcg_cfg_keyword", "kcg_dtype_size", "kcg_check_config", "kcg_select_kind", "kcg_kernel_name",
     "kcg_launch_dims", "kcg_reference_lds_bytes", "kcg_block_mapping", "kcg_compile_matmul",
     "kcg_instantiation_source", "kcg_load", "kcg_launch", "kcg_benchmark", "kcg_unload",
-    "kcg_device_info", "kcg_last_error", "kcg_version",
+    "kcg_device_info", "kcg_last_error", "kcg_version", "kcg_compile_matmul_ex", "kcg_launch_batched",
 )
 
 _lib = None
@@ -120,6 +121,10 @@ def lib():
                                 ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64,
                                 ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                 ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
+    L.kcg_compile_matmul_ex.argtypes = [cfgp, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(KernelInfo)]
+    L.kcg_launch_batched.argtypes = [ctypes.c_uint64, i32p, i32p, ctypes.c_int, ctypes.c_uint64,
+                                     ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int32,
+                                     ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_float, ctypes.c_float]
     L.kcg_unload.argtypes = [ctypes.c_uint64]
     L.kcg_device_info.argtypes = [ctypes.c_int, i32p, i32p, i32p, ctypes.c_char_p, ctypes.c_int]
     _lib = L
@@ -209,11 +214,16 @@ def instantiation_source(values, kind=KIND_AUTO):
     return buf.value.decode()
 
 
-def compile_matmul(values, arch="gfx950", kind=KIND_AUTO):
-    """-> dict(code_path, kernel_name, grid, block, lds_bytes, kind, cache_hit)"""
+def compile_matmul(values, arch="gfx950", kind=KIND_AUTO, epilogue=None):
+    """-> dict(code_path, kernel_name, grid, block, lds_bytes, kind, cache_hit).
+    epilogue None: the reference's three-pointer kernel; EPILOGUE_NONE / EPILOGUE_ALPHA_BETA: the
+    batched-strided kernel form (launch it with launch_batched)."""
     c = make_cfg(values)
     info = KernelInfo()
-    check(lib().kcg_compile_matmul(ctypes.byref(c), arch.encode(), kind, ctypes.byref(info)))
+    if epilogue is None:
+        check(lib().kcg_compile_matmul(ctypes.byref(c), arch.encode(), kind, ctypes.byref(info)))
+    else:
+        check(lib().kcg_compile_matmul_ex(ctypes.byref(c), arch.encode(), kind, int(epilogue), ctypes.byref(info)))
     return {
         "code_path": info.code_path.decode(),
         "kernel_name": info.kernel_name.decode(),
@@ -235,6 +245,11 @@ def load(code_path, kernel_name_, lds_bytes, device):
 
 def launch(function, grid, block, lds_bytes, stream, a, b, c):
     check(lib().kcg_launch(function, _dims(grid), _dims(block), int(lds_bytes), int(stream), int(a), int(b), int(c)))
+
+
+def launch_batched(function, grid, block, lds_bytes, stream, a, b, c, batch, stride_a, stride_b, stride_c, alpha=1.0, beta=0.0):
+    check(lib().kcg_launch_batched(function, _dims(grid), _dims(block), int(lds_bytes), int(stream), int(a), int(b), int(c),
+                                   int(batch), int(stride_a), int(stride_b), int(stride_c), float(alpha), float(beta)))
 
 
 def benchmark(function, grid, block, lds_bytes, stream, a, b, c, warmup=1, iters=20, reps=0):

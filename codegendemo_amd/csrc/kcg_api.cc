@@ -419,6 +419,11 @@ static long code_object_scratch_bytes(const std::vector<char>& code) {
     if (left >= 2 && p[0] == 0xcc) return p[1];
     if (left >= 3 && p[0] == 0xcd) return (p[1] << 8) | p[2];
     if (left >= 5 && p[0] == 0xce) return ((long)p[1] << 24) | (p[2] << 16) | (p[3] << 8) | p[4];
+    if (left >= 9 && p[0] == 0xcf) {
+      long v = 0;
+      for (int b = 1; b <= 8; ++b) v = (v << 8) | p[b];
+      return v;
+    }
   }
   return -1;
 }
@@ -428,11 +433,12 @@ static const int kBuildSpills = 1;
 
 // Builds (or finds in the cache) the code object of config c as kernel family k; `allow_direct` lets a
 // matrix-core config that is eligible for direct global->LDS staging use that kernel.
-static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, const std::string& arch, kcg_kernel_info* out) {
+// ex < 0: the reference's three-pointer kernel; 0 / 1: the batched-strided form without / with alpha-beta.
+static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, const std::string& arch, int ex, kcg_kernel_info* out) {
   const bool xcd = env_flag("KCG_XCD_REMAP", true);
   const bool direct = allow_direct && k == KCG_KIND_MFMA && kcg::mfma_direct(c);
-  const std::string name = kcg::kernel_name(c);
-  const std::string stub = kcg::instantiation_source(c, k, xcd, allow_direct);
+  const std::string name = ex < 0 ? kcg::kernel_name(c) : kcg::kernel_name_ex(c, ex);
+  const std::string stub = kcg::instantiation_source(c, k, xcd, allow_direct, ex);
 
   memset(out, 0, sizeof(*out));
   if (name.size() >= sizeof(out->kernel_name)) return fail(KCG_ERR_ARGUMENT, "kernel name too long");
@@ -506,7 +512,8 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
   // The direct-staging kernel reads LDS with instructions the compiler does not know to be
   // asynchronous: a fragment register spilled to scratch memory would be stored before its data has
   // arrived.  Such a build is never used (nor cached): the caller falls back to register staging.
-  if (direct && code_object_scratch_bytes(code) > 0) {
+  // (a code object whose metadata does not say counts as spilling: the kernel is not used unverified)
+  if (direct && code_object_scratch_bytes(code) != 0) {
     const char note[] = "direct-staging build needs scratch memory (register spills); register staging is used instead\n";
     write_file_atomic(spill_marker, note, sizeof(note) - 1);
     return kBuildSpills;
@@ -527,8 +534,21 @@ int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind,
   int k = resolve_kind(c, kind, &why);
   if (k < 0) return fail(k, "invalid config: " + why);
   const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
-  int r = build_variant(c, k, /*allow_direct=*/true, arch, out);
-  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, out);
+  int r = build_variant(c, k, /*allow_direct=*/true, arch, -1, out);
+  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, -1, out);
+  return r;
+}
+
+int kcg_compile_matmul_ex(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, int epilogue, kcg_kernel_info* out) {
+  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
+  if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_ALPHA_BETA) return fail(KCG_ERR_ARGUMENT, "unknown epilogue");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  std::string why;
+  int k = resolve_kind(c, kind, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
+  int r = build_variant(c, k, /*allow_direct=*/true, arch, epilogue, out);
+  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, epilogue, out);
   return r;
 }
 
@@ -580,6 +600,27 @@ int kcg_launch(uint64_t function, const int32_t grid[3], const int32_t block[3],
   HIP_READY();
   HIP_TRY(HIPF(hipModuleLaunchKernel)((hipFunction_t)(uintptr_t)function, grid[0], grid[1], grid[2], block[0], block[1],
                                 block[2], lds_bytes, (hipStream_t)(uintptr_t)stream, params, nullptr));
+  return KCG_OK;
+}
+
+int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes, uint64_t stream,
+                       uint64_t a, uint64_t b, uint64_t c, int32_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                       float alpha, float beta) {
+  if (!function || !grid || !block) return fail(KCG_ERR_ARGUMENT, "null function / dims");
+  if (batch < 0 || batch > 65535) return fail(KCG_ERR_ARGUMENT, "batch must be in [0, 65535]");
+  if (stride_a < 0 || stride_b < 0 || stride_c < 0) return fail(KCG_ERR_ARGUMENT, "strides must not be negative");
+  if (batch > 1 && stride_c == 0) return fail(KCG_ERR_ARGUMENT, "stride_c = 0 would make the problems of a batch write the same C");
+  if ((int64_t)grid[0] * grid[1] * grid[2] <= 0 || batch == 0) return KCG_OK;  // nothing to do
+  if (grid[1] != 1 || grid[2] != 1) return fail(KCG_ERR_ARGUMENT, "the batch goes on grid[1]: grid must be {n, 1, 1}");
+  if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
+  void* pa = (void*)(uintptr_t)a;
+  void* pb = (void*)(uintptr_t)b;
+  void* pc = (void*)(uintptr_t)c;
+  long sa = (long)stride_a, sb = (long)stride_b, sc = (long)stride_c;
+  void* params[8] = {&pa, &pb, &pc, &sa, &sb, &sc, &alpha, &beta};
+  HIP_READY();
+  HIP_TRY(HIPF(hipModuleLaunchKernel)((hipFunction_t)(uintptr_t)function, grid[0], batch, 1, block[0], block[1], block[2],
+                                lds_bytes, (hipStream_t)(uintptr_t)stream, params, nullptr));
   return KCG_OK;
 }
 

@@ -1,6 +1,7 @@
 // kcg_config.cc — see kcg_config.h.
 #include "kcg_config.h"
 
+#include <cstdlib>
 #include <sstream>
 
 namespace kcg {
@@ -263,11 +264,23 @@ int lds_bytes(const MatmulConfig& c, int kind, bool allow_direct) {
   return (r + 15) & ~15;
 }
 
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  const int x = atoi(v);
+  return x > 0 ? x : dflt;
+}
+// An MI355X in its default (single-partition) mode: 256 compute units in 8 XCDs.  Another partition mode
+// (or another part) is described with $KCG_NUM_CUS / $KCG_NUM_XCDS; both are baked into the instantiation.
+int num_cus() { return env_int("KCG_NUM_CUS", 256); }
+int num_xcds() { return env_int("KCG_NUM_XCDS", 8); }
+
 // Rewriter::BlockMapping with isCol=true (Rewriter.cc:726-761; Rewriter.h:112)
 void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int* bx) {
   const int gy = c.grid_y(), gx = c.grid_x();
   const int nb = gy * gx;
-  if (xcd_remap && nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
+  const int nx = num_xcds();
+  if (xcd_remap && nx > 1 && nb % nx == 0) bid = (bid % nx) * (nb / nx) + bid / nx;
   const int g = c.BLOCK_MAPPING;
   if (g > 0 && gy % g == 0) {
     const int gn = g * gx;
@@ -279,7 +292,11 @@ void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int*
   }
 }
 
-std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap, bool allow_direct) {
+std::string kernel_name_ex(const MatmulConfig& c, int epilogue) {
+  return kernel_name(c) + (epilogue ? "EXab_" : "EX_");
+}
+
+std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap, bool allow_direct, int ex) {
   std::ostringstream s;
   const char* acc = (c.dtC == KCG_DT_FLOAT64) ? "double" : "float";
   s << "// generated by libkcg_gemm: instantiation of the " << (kind == KCG_KIND_MFMA ? "gemm_mfma" : "gemm_simt")
@@ -303,15 +320,29 @@ std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap
   Bv("ATRANS", c.ATRANS != 0);
   Bv("EDGE", c.edge());
   Bv("XCD_REMAP", xcd_remap);
+  I("NUM_CU", num_cus()); I("NUM_XCD", num_xcds());
+  Bv("EPI", ex > 0);
   Bv("DIRECT_ELIGIBLE", kind == KCG_KIND_MFMA && mfma_direct(c));   // the rule; the device header re-derives and compares it
   Bv("DIRECT", allow_direct && kind == KCG_KIND_MFMA && mfma_direct(c));
   I("SIMT_PAD_A", simt_pad_a(c)); I("SIMT_PAD_B", 0);
   s << "};\n}  // namespace\n\n";
-  s << "extern \"C\" __global__ __launch_bounds__(" << c.thread_num() << ") void " << kernel_name(c)
-    << "(const Cfg::TA* __restrict__ A, const Cfg::TB* __restrict__ B, Cfg::TC* __restrict__ C) {\n";
-  s << "  extern __shared__ __attribute__((aligned(16))) char kcg_shm0[];\n";
-  s << "  kcg::" << (kind == KCG_KIND_MFMA ? "gemm_mfma" : "gemm_simt") << "<Cfg>(A, B, C, kcg_shm0);\n";
-  s << "}\n";
+  const char* fn = kind == KCG_KIND_MFMA ? "gemm_mfma" : "gemm_simt";
+  if (ex < 0) {
+    s << "extern \"C\" __global__ __launch_bounds__(" << c.thread_num() << ") void " << kernel_name(c)
+      << "(const Cfg::TA* __restrict__ A, const Cfg::TB* __restrict__ B, Cfg::TC* __restrict__ C) {\n";
+    s << "  extern __shared__ __attribute__((aligned(16))) char kcg_shm0[];\n";
+    s << "  kcg::" << fn << "<Cfg>(A, B, C, kcg_shm0);\n";
+    s << "}\n";
+  } else {
+    // batched / strided form: problem blockIdx.y of the batch lives stride_* elements further in each
+    // buffer; alpha and beta are used only by an instantiation with the alpha/beta epilogue
+    s << "extern \"C\" __global__ __launch_bounds__(" << c.thread_num() << ") void " << kernel_name_ex(c, ex)
+      << "(const Cfg::TA* A, const Cfg::TB* B, Cfg::TC* C, long stride_a, long stride_b, long stride_c, float alpha, float beta) {\n";
+    s << "  extern __shared__ __attribute__((aligned(16))) char kcg_shm0[];\n";
+    s << "  const long z = blockIdx.y;\n";
+    s << "  kcg::" << fn << "<Cfg>(A + z * stride_a, B + z * stride_b, C + z * stride_c, kcg_shm0, kcg::EpiArgs{alpha, beta});\n";
+    s << "}\n";
+  }
   return s.str();
 }
 

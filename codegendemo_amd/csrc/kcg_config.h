@@ -57,8 +57,13 @@ bool mfma_direct(const MatmulConfig& c);      // matrix-core kernel stages opera
 int lds_bytes(const MatmulConfig& c, int kind, bool allow_direct = true);  // what the chosen kernel really needs
 void block_mapping(const MatmulConfig& c, int bid, bool xcd_remap, int* by, int* bx);
 
-// HIP text of the instantiation stub for (config, kind, xcd_remap).
-std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap, bool allow_direct = true);
+int num_cus();    // compute units / XCDs of the (partition of the) GPU the kernels are built for: 256 / 8,
+int num_xcds();   // or $KCG_NUM_CUS / $KCG_NUM_XCDS
+
+// HIP text of the instantiation stub for (config, kind, xcd_remap).  ex < 0: the reference's kernel form (three
+// pointers); ex = 0 / 1: the batched-strided form, without / with the alpha-beta epilogue (kernel_name_ex).
+std::string instantiation_source(const MatmulConfig& c, int kind, bool xcd_remap, bool allow_direct = true, int ex = -1);
+std::string kernel_name_ex(const MatmulConfig& c, int epilogue);
 
 constexpr int kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KiB LDS per CU, one workgroup may take all
 constexpr int kMaxThreads = 1024;

@@ -51,21 +51,28 @@ __device__ __forceinline__ void copy_bytes(void* dst, const void* src) {
   typedef typename RawVec<NBYTES>::type V;
   *reinterpret_cast<V*>(dst) = *reinterpret_cast<const V*>(src);
 }
+// the same with a non-temporal store (streaming data that the kernel does not read again)
+template <int NBYTES>
+__device__ __forceinline__ void copy_bytes_nt(void* dst, const void* src) {
+  typedef typename RawVec<NBYTES>::type V;
+  __builtin_nontemporal_store(*reinterpret_cast<const V*>(src), reinterpret_cast<V*>(dst));
+}
 
 // ---------------------------------------------------------------------------------------------
 // Block id -> (by, bx).  Rewriter::BlockMapping (Rewriter.cc:726-761): groups of BLOCK_MAPPING block
 // rows are walked column by column so that concurrently resident blocks share B panels in L2.
-// On top of it, when the block count is a multiple of 8, consecutive hardware ids (which the
-// dispatcher deals round-robin to the 8 XCDs, each with a private L2) are remapped so that every XCD
-// walks one contiguous eighth of that order.
+// On top of it, when the block count is a multiple of the number of XCDs (C::NUM_XCD, 8 on an MI355X),
+// consecutive hardware ids (which the dispatcher deals round-robin to the XCDs, each with a private L2)
+// are remapped so that every XCD walks one contiguous part of that order.
 // ---------------------------------------------------------------------------------------------
 template <class C>
 __device__ __forceinline__ void block_coords(int bid, int& by, int& bx) {
   constexpr int GY = cdiv(C::M, C::BM);
   constexpr int GX = cdiv(C::N, C::BN);
   constexpr int NB = GY * GX;
-  if constexpr (C::XCD_REMAP && (NB % 8 == 0)) {
-    bid = (bid % 8) * (NB / 8) + bid / 8;
+  constexpr int NX = C::NUM_XCD;
+  if constexpr (C::XCD_REMAP && NX > 1 && (NB % NX == 0)) {
+    bid = (bid % NX) * (NB / NX) + bid / NX;
   }
   if constexpr (C::BLOCK_MAPPING > 0 && (GY % (C::BLOCK_MAPPING > 0 ? C::BLOCK_MAPPING : 1) == 0)) {
     constexpr int G = C::BLOCK_MAPPING;
@@ -158,13 +165,15 @@ __device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r,
 }
 
 // Store VEC consecutive output elements (converted from the accumulator type) with the same rules.
-template <class TC, class ACC, int VEC, bool EDGE, bool ALIGNED>
+template <class TC, class ACC, int VEC, bool EDGE, bool ALIGNED, bool NT = false>
 __device__ __forceinline__ void gstore(TC* __restrict__ base, const ACC* src, int r, int c, int LD, int RMAX, int CMAX) {
   TC tmp[VEC];
 #pragma unroll
   for (int e = 0; e < VEC; ++e) tmp[e] = (TC)src[e];
   if constexpr (!EDGE) {
-    if constexpr (ALIGNED) {
+    if constexpr (ALIGNED && NT) {
+      copy_bytes_nt<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
+    } else if constexpr (ALIGNED) {
       copy_bytes<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
     } else {
 #pragma unroll
@@ -179,13 +188,33 @@ __device__ __forceinline__ void gstore(TC* __restrict__ base, const ACC* src, in
   }
 }
 
+// Epilogue C = alpha * (A B) + beta * C (the call shape of the vendor sgemm the reference profiles against,
+// runRoc.cpp:27-28,53-66), compiled in only when the instantiation asks for it (C::EPI).  As in BLAS, beta == 0
+// means that C is not read at all (whatever it held, NaN included, does not reach the result).
+struct EpiArgs {
+  float alpha, beta;
+};
+template <class TC, class ACC, int VEC, bool EDGE, bool ALIGNED>
+__device__ __forceinline__ void epi_apply(ACC* v, const TC* base, int r, int c, int LD, int RMAX, int CMAX, EpiArgs ep) {
+  const ACC alpha = (ACC)ep.alpha, beta = (ACC)ep.beta;
+  if (ep.beta != 0.f) {
+    TC old[VEC];
+    gload<TC, VEC, EDGE, ALIGNED>(old, base, r, c, LD, RMAX, CMAX);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = alpha * v[e] + beta * (ACC)old[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = alpha * v[e];
+  }
+}
+
 // Split-U epilogue shared by both families (Rewriter::splitUReduce / splitUWrite, Rewriter.cc:603-663):
 // smC is [LSU][BM][BN] accumulators; slice 0 is copied, slices 1..LSU-1 are added in order, and the
 // sum is written to C with GLOB_STORE_WIDTH-wide vectors using the (non-)continuous map selected by
 // REDUCE_C_CONTINUOUS (Optimizer.cc:241-282).
 template <class C, int NT>
 __device__ __forceinline__ void splitu_reduce_store(typename C::TC* __restrict__ Cm, const typename C::ACC* smC,
-                                                    int tid, int m0, int n0) {
+                                                    int tid, int m0, int n0, EpiArgs ep) {
   typedef typename C::ACC ACC;
   constexpr int GSW = C::GSW;
   constexpr bool CONT = C::RC != 0 || (NT % C::BM != 0) || (C::BN % ((NT / C::BM) * GSW) != 0);
@@ -203,6 +232,7 @@ __device__ __forceinline__ void splitu_reduce_store(typename C::TC* __restrict__
 #pragma unroll
         for (int e = 0; e < GSW; ++e) sum[e] += smC[(z * C::BM + r) * C::BN + c + e];
       }
+      if constexpr (C::EPI) epi_apply<typename C::TC, ACC, GSW, C::EDGE, ALIGNED>(sum, Cm, m0 + r, n0 + c, C::N, C::M, C::N, ep);
       gstore<typename C::TC, ACC, GSW, C::EDGE, ALIGNED>(Cm, sum, m0 + r, n0 + c, C::N, C::M, C::N);
     }
   }

@@ -6,6 +6,45 @@
 
 namespace kcg {
 
+// ---------------------------------------------------------------------------------------------
+// In-kernel time line (diagnostic build, -DKCG_TIMELINE=1 or 2 through $KCG_EXTRA_FLAGS; 0 = off, no
+// code).  Every wave of gemm_mfma_direct then writes one record of KCG_TL_WORDS 64-bit words to the buffer
+// whose address the host has stored in the module's global `kcg_timeline_ptr` (hipModuleGetGlobal),
+// record index = block * waves + wave:
+//   [0] block start  [1] first K tile has landed  [2] K loop done  [3] C stores issued
+//   [4] C stores acknowledged                    (constant 100 MHz clock, 10 ns units)
+//   [5] shader-clock cycles spent in the K loop
+//   [6] HW_ID (low half) and XCC_ID (high half) registers: which compute unit / XCD the wave ran on
+//   [7] level 2 only: shader-clock cycles this wave spent between asking for and passing the K-loop
+//       barriers (wait for its own fetches + LDS reads + the other waves); costs one extra scalar-memory
+//       round trip per K tile, so the times of level 2 are a little longer than those of level 1
+// kcg_runner --timeline builds such a kernel, runs it and prints the per-phase budget.
+// ---------------------------------------------------------------------------------------------
+#ifndef KCG_TIMELINE
+#define KCG_TIMELINE 0
+#endif
+// 1: the direct-staging kernel writes C with non-temporal stores (C is written once and not read again by
+// the kernel: the stores need not displace operand panels from L2)
+#ifndef KCG_C_NT
+#define KCG_C_NT 0
+#endif
+#if KCG_TIMELINE
+#define KCG_TL_WORDS 8
+extern "C" {
+__device__ unsigned long long* kcg_timeline_ptr = nullptr;
+}
+__device__ __forceinline__ unsigned long long tl_realtime() {
+  unsigned long long t;
+  asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t)::"memory");
+  return t;
+}
+__device__ __forceinline__ unsigned long long tl_cycles() {
+  unsigned long long t;
+  asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t)::"memory");
+  return t;
+}
+#endif
+
 // =============================================================================================
 // Family 2b: matrix-core kernel with direct global->LDS staging.
 //
@@ -107,7 +146,7 @@ struct DirectPlan {
   static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
   static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
   // Two blocks on a compute unit beat one block with deeper staging when the launch has more blocks than the
-  // chip has compute units (256): one block's prologue, barrier waits and C stores run under the other's
+  // chip has compute units (C::NUM_CU): one block's prologue, barrier waits and C stores run under the other's
   // matrix work (measured 2-5 % at 4096x1536x1000, 2048^3 and 4096^3 with 128x64 and 128x128 tiles).  Where
   // two blocks fit the register file (512 registers per lane and SIMD, a block's waves dealt evenly over
   // the four SIMDs: a wave holds WM*WN/64 accumulators and some 64 registers of fragments and addresses) the
@@ -116,7 +155,7 @@ struct DirectPlan {
 #define KCG_DIRECT_NST 0              /* upper limit of the number of LDS stages; 0: the rule below */
 #endif
   static constexpr int GRID_BLOCKS = ((C::M + C::BM - 1) / C::BM) * ((C::N + C::BN - 1) / C::BN);
-  static constexpr bool PAIR = GRID_BLOCKS > 256 && NW % 4 == 0 && (WM * WN / 64 + 64) * (NW / 2) <= 512 &&
+  static constexpr bool PAIR = GRID_BLOCKS > C::NUM_CU && NW % 4 == 0 && (WM * WN / 64 + 64) * (NW / 2) <= 512 &&
                                2 * STAGE_BYTES <= 80 * 1024;
   static constexpr int NST_LIMIT = KCG_DIRECT_NST > 0 ? KCG_DIRECT_NST : (PAIR ? (80 * 1024) / STAGE_BYTES : 4);
   static constexpr int NST_TOP = NST_LIMIT > 4 ? 4 : NST_LIMIT;
@@ -131,7 +170,7 @@ struct DirectPlan {
 
 template <class C>
 __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
-                                                 typename C::TC* __restrict__ Cm, char* smem) {
+                                                 typename C::TC* __restrict__ Cm, char* smem, EpiArgs ep = EpiArgs{1.f, 0.f}) {
   typedef typename C::TA T;
   typedef typename C::TC TC;
   typedef DirectPlan<C> P;
@@ -164,6 +203,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   int by, bx;
   block_coords<C>(blockIdx.x, by, bx);
   const int m0 = by * BM, n0 = bx * BN;
+#if KCG_TIMELINE
+  unsigned long long tl[KCG_TL_WORDS] = {};
+  tl[0] = tl_realtime();
+#endif
 
   // One LDS array holds the NST stages.  (No LDS access of this kernel is visible to the compiler as a
   // load: otherwise it would have to assume that the load may touch a stage a fetch is in flight to
@@ -441,6 +484,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();                                            // ... and everyone's (bare barrier: see the K loop)
   asm volatile("" ::: "memory");
+#if KCG_TIMELINE
+  tl[1] = tl_realtime();
+  const unsigned long long tl_c0 = tl_cycles();
+#endif
   FragA fa[TMI];
   FragB fb[2][TNI];
   static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
@@ -484,6 +531,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         if constexpr (LAST && I == RB) {
           // tile kt+1 has landed (this wave's part): of the fetches issued so far only those of the
           // tiles behind it may still be in flight
+#if KCG_TIMELINE >= 2
+          wait_lds();        // (level 2: the stamp's own wait must not count as barrier wait)
+          const unsigned long long tl_b0 = tl_cycles();
+#endif
           if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
           wait_lds();        // this wave's reads of stage CUR have all returned
           // ... everyone's part; and every wave is done reading stage CUR.  The bare barrier instruction:
@@ -493,6 +544,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           asm volatile("" ::: "memory");
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
+#if KCG_TIMELINE >= 2
+          tl[7] += tl_cycles() - tl_b0;
+#endif
         }
         // the empty asm statements make the fragments "outputs" of the wait: the matrix-core
         // instructions that consume them cannot be scheduled in front of it
@@ -568,6 +622,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // the last matrix-core results must have left the pipeline before the epilogue reads them (the
   // compiler, which normally inserts these wait states, does not know the instructions above)
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#if KCG_TIMELINE
+  tl[5] = tl_cycles() - tl_c0;
+  tl[2] = tl_realtime();
+#endif
   // ... and the epilogue's reads must stay behind those wait states: an accumulator is an ordinary
   // register value to the compiler, free to be read (converted, moved) ahead of an asm statement that does
   // not mention it.  Passing every accumulator through an empty asm statement behind the wait states
@@ -582,8 +640,15 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int NACC = (int)(sizeof(Acc) / sizeof(float));
   const int orow = lane % MF;
   const int ocol = (lane / MF) * 4;
+  // Diagnostic builds only (never set by the library itself): -DKCG_DIAG_STORE_ROWS=n stores just the first n
+  // rows of matrix-core tiles of every wave tile, so C is INCOMPLETE; timing such a build shows how much of a
+  // launch the C stores cost (n = 0) and what hiding a part of them under matrix work could gain at best.
+#ifndef KCG_DIAG_STORE_ROWS
+#define KCG_DIAG_STORE_ROWS -1
+#endif
+  constexpr int STORE_ROWS = KCG_DIAG_STORE_ROWS < 0 ? TMI : cmin(TMI, KCG_DIAG_STORE_ROWS);
 #pragma unroll
-  for (int i = 0; i < TMI; ++i)
+  for (int i = 0; i < STORE_ROWS; ++i)
 #pragma unroll
     for (int j = 0; j < TNI; ++j)
 #pragma unroll
@@ -593,8 +658,22 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-        gstore<TC, float, 4, (EDGE_M || EDGE_N), true>(Cm, v, row, col, N, M, N);
+        if constexpr (C::EPI) epi_apply<TC, float, 4, (EDGE_M || EDGE_N), true>(v, Cm, row, col, N, M, N, ep);
+        gstore<TC, float, 4, (EDGE_M || EDGE_N), true, (KCG_C_NT != 0)>(Cm, v, row, col, N, M, N);
       }
+#if KCG_TIMELINE
+  asm volatile("" ::: "memory");
+  tl[3] = tl_realtime();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  tl[4] = tl_realtime();
+  tl[6] = (unsigned long long)__builtin_amdgcn_s_getreg(4 | (31 << 11)) |            // HW_REG_HW_ID
+          ((unsigned long long)__builtin_amdgcn_s_getreg(20 | (31 << 11)) << 32);     // HW_REG_XCC_ID
+  if (kcg_timeline_ptr != nullptr && lane == 0) {
+    unsigned long long* rec = kcg_timeline_ptr + ((size_t)blockIdx.x * NW + wave) * KCG_TL_WORDS;
+#pragma unroll
+    for (int w = 0; w < KCG_TL_WORDS; ++w) rec[w] = tl[w];
+  }
+#endif
 }
 
 }  // namespace kcg

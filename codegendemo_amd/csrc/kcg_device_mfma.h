@@ -12,9 +12,9 @@ namespace kcg {
 // =============================================================================================
 template <class C>
 __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
-                                          typename C::TC* __restrict__ Cm, char* smem) {
+                                          typename C::TC* __restrict__ Cm, char* smem, EpiArgs ep = EpiArgs{1.f, 0.f}) {
   if constexpr (DirectPlan<C>::OK) {
-    gemm_mfma_direct<C>(A, B, Cm, smem);
+    gemm_mfma_direct<C>(A, B, Cm, smem, ep);
     return;
   }
   typedef typename C::TA T;   // TA == TB for this family
@@ -299,7 +299,7 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
           smC[(wz * BM + row) * BN + col] = acc[i][j][e];
         }
     __syncthreads();
-    splitu_reduce_store<C, NT>(Cm, smC, tid, m0, n0);
+    splitu_reduce_store<C, NT>(Cm, smC, tid, m0, n0, ep);
   } else {
 #pragma unroll
     for (int i = 0; i < TMI; ++i)
@@ -309,7 +309,11 @@ __device__ __forceinline__ void gemm_mfma(const typename C::TA* __restrict__ A, 
         for (int e = 0; e < NACC; ++e) {
           const int row = m0 + wy * WM + i * MF + acc_row(e);
           const int col = n0 + wx * WN + j * MF + ocol;
-          if (!EDGE || (row < M && col < N)) Cm[(long)row * N + col] = (TC)acc[i][j][e];
+          if (!EDGE || (row < M && col < N)) {
+            AccT v = acc[i][j][e];
+            if constexpr (C::EPI) epi_apply<TC, AccT, 1, false, true>(&v, Cm, row, col, N, M, N, ep);
+            Cm[(long)row * N + col] = (TC)v;
+          }
         }
   }
 }

@@ -9,7 +9,7 @@ namespace kcg {
 // =============================================================================================
 template <class C>
 __device__ __forceinline__ void gemm_simt(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
-                                          typename C::TC* __restrict__ Cm, char* smem) {
+                                          typename C::TC* __restrict__ Cm, char* smem, EpiArgs ep = EpiArgs{1.f, 0.f}) {
   typedef typename C::TA TA;
   typedef typename C::TB TB;
   typedef typename C::TC TC;
@@ -200,7 +200,7 @@ __device__ __forceinline__ void gemm_simt(const typename C::TA* __restrict__ A, 
             }
         }
     __syncthreads();
-    splitu_reduce_store<C, NT>(Cm, smC, tid, m0, n0);
+    splitu_reduce_store<C, NT>(Cm, smC, tid, m0, n0, ep);
   } else {
     // direct store, TSW_B-wide pieces (Optimizer.cc:193-215,412-421)
     constexpr bool AL_C = (N % C::TSW_B == 0);
@@ -218,6 +218,7 @@ __device__ __forceinline__ void gemm_simt(const typename C::TA* __restrict__ A, 
             for (int j1 = 0; j1 < WRB; ++j1) {
               const int col = (j0 * C::BLN + warp_x) * C::WLN * C::WSW_B + (j1 * C::WLN + lane_x) * C::TSW_B;
               const int rj = j0 * C::WSW_B + j1 * C::TSW_B;
+              if constexpr (C::EPI) epi_apply<TC, ACC, C::TSW_B, EDGE, AL_C>(&acc[ri][rj], Cm, m0 + row, n0 + col, N, M, N, ep);
               gstore<TC, ACC, C::TSW_B, EDGE, AL_C>(Cm, &acc[ri][rj], m0 + row, n0 + col, N, M, N);
             }
         }

@@ -6,9 +6,16 @@
 // print, naive `gemm_kernel` + `verify_kernel`, matmul.cpp:2327-2348,2386-2553).
 //
 //   kcg_runner --config <file.json> [--index i] [--kind auto|simt|mfma] [--iters n] [--tol t]
+//              [--dist uniform|normal] [--timeline 1|2]
 //       compiles entry i of a {"cfgs": [...]} file (or a single flat config object) through
 //       libkcg_gemm.so, loads it, verifies it against the naive kernel and times it
-//       (--compile-only 1 stops after the compile: fills the code-object cache on a host without a GPU)
+//       (--compile-only 1 stops after the compile: fills the code-object cache on a host without a GPU).
+//       --dist: operands uniform on [-1,1) (default) or normal(0, 0.5), the distribution the 16-bit
+//       benchmark uses (on a power-limited part the speed of a matrix-core kernel depends on the data).
+//       --timeline: builds the direct-staging kernel with its in-kernel time stamps (-DKCG_TIMELINE=level
+//       added to $KCG_EXTRA_FLAGS), runs it back to back and prints where the time of one launch goes:
+//       block start, first K tile landed, K loop done, C stores issued / acknowledged, per XCD and over
+//       all waves, the shader clock during the K loop, and the gap to the next launch.
 //   kcg_runner M N K gridX blockX <code-object> <kernel-name> [ldsBytes] [dtypeCode] [isATrans]
 //       the reference runner's argument list (runkernel.cpp:63-66): launches an existing code object
 //
@@ -227,6 +234,25 @@ __global__ __launch_bounds__(256) void write_only(float4* __restrict__ out, size
   for (size_t i = threadIdx.x; i < per_block; i += 256) p[i] = v;
 }
 
+// the C stores of a 256 x 256 x (4 waves of 128 x 128) GEMM epilogue and nothing else: block b owns tile
+// (b / 16, b % 16) of a 4096 x 4096 fp32 matrix.  LINE = 64: every store instruction of a wave writes 16 rows x
+// 64 contiguous bytes (what 16x16 accumulator tiles give); LINE = 128: 8 rows x 128 bytes (whole cache
+// lines per row).  NT: non-temporal stores.
+template <int LINE, bool NT>
+__global__ __launch_bounds__(256) void write_tiles(float* __restrict__ out) {
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int row0 = (blockIdx.x / 16) * 256 + (wave / 2) * 128, col0 = (blockIdx.x % 16) * 256 + (wave % 2) * 128;
+  constexpr int LPR = LINE / 16, RPI = 64 / LPR;       // lanes per row, rows per instruction
+  typedef float v4 __attribute__((ext_vector_type(4)));
+  const v4 v = {1.f, 2.f, 3.f, 4.f};
+  for (int r = 0; r < 128; r += RPI)
+    for (int c = 0; c < 128; c += LINE / 4) {
+      v4* p = (v4*)(out + (size_t)(row0 + r + lane / LPR) * 4096 + col0 + c + (lane % LPR) * 4);
+      if constexpr (NT) __builtin_nontemporal_store(v, p);
+      else *p = v;
+    }
+}
+
 template <class F>
 static double launch_period_us(F launch, int n) {
   for (int i = 0; i < 200; ++i) launch();
@@ -251,9 +277,15 @@ static int launch_cost_main() {
   const double e256 = launch_period_us([&] { hipLaunchKernelGGL(empty_kernel, dim3(256), dim3(256), 0, 0, sink); }, n);
   const double elds = launch_period_us([&] { hipLaunchKernelGGL((empty_kernel_lds<65536>), dim3(256), dim3(256), 0, 0, sink); }, n);
   const double w = launch_period_us([&] { hipLaunchKernelGGL(write_only, dim3(256), dim3(256), 0, 0, (float4*)sink, bytes / 16 / 256); }, 500);
+  const double t64 = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<64, false>), dim3(256), dim3(256), 0, 0, sink); }, 500);
+  const double t128 = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<128, false>), dim3(256), dim3(256), 0, 0, sink); }, 500);
+  const double t64nt = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<64, true>), dim3(256), dim3(256), 0, 0, sink); }, 500);
+  const double t128nt = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<128, true>), dim3(256), dim3(256), 0, 0, sink); }, 500);
   printf("{\"launch_cost\": {\"period_us\": {\"empty_1_block\": %.2f, \"empty_256_blocks\": %.2f, \"empty_256_blocks_64KiB_lds\": %.2f, "
-         "\"write_64MiB\": %.2f}, \"write_GBps\": %.0f, \"note\": \"back-to-back launches on one stream, HIP events around the whole run\"}}\n",
-         e1, e256, elds, w, bytes / (w - e256) * 1e-3);
+         "\"write_64MiB\": %.2f, \"write_64MiB_as_gemm_tiles_64B_per_row\": %.2f, \"write_64MiB_as_gemm_tiles_128B_per_row\": %.2f, "
+         "\"same_64B_nontemporal\": %.2f, \"same_128B_nontemporal\": %.2f}, \"write_GBps\": %.0f, "
+         "\"note\": \"back-to-back launches on one stream, HIP events around the whole run\"}}\n",
+         e1, e256, elds, w, t64, t128, t64nt, t128nt, bytes / (w - e256) * 1e-3);
   HIP_OK(hipFree(sink));
   return 0;
 }
@@ -261,6 +293,14 @@ static int launch_cost_main() {
 static float lcg_uniform(uint64_t& s) {   // [-1, 1)
   s = s * 6364136223846793005ull + 1442695040888963407ull;
   return (float)((int32_t)(s >> 40) - (1 << 23)) / (float)(1 << 23);
+}
+
+static float lcg_normal(uint64_t& st, float std) {   // Box-Muller on two uniforms
+  st = st * 6364136223846793005ull + 1442695040888963407ull;
+  const float u1 = ((float)(st >> 40) + 1.0f) / 16777217.0f;
+  st = st * 6364136223846793005ull + 1442695040888963407ull;
+  const float u2 = (float)(st >> 40) / 16777216.0f;
+  return sqrtf(-2.0f * logf(u1)) * cosf(6.2831853f * u2) * std;
 }
 
 template <class T>
@@ -271,6 +311,69 @@ static void* upload(const std::vector<float>& h) {
   HIP_OK(hipMalloc(&d, t.size() * sizeof(T)));
   HIP_OK(hipMemcpy(d, t.data(), t.size() * sizeof(T), hipMemcpyHostToDevice));
   return d;
+}
+
+// ---- where the time of one launch goes: reads the records a -DKCG_TIMELINE kernel writes (layout: see
+// kcg_device_direct.h) for the last of `launches` back-to-back launches -----------------------------
+static int timeline_report(uint64_t module, uint64_t function, const kcg_kernel_info& info, int waves_per_block,
+                           uint64_t dA, uint64_t dB, uint64_t dC, double flops, int level) {
+  const int TLW = 8;
+  const size_t nrec = (size_t)info.grid[0] * waves_per_block;
+  unsigned long long* d_rec;
+  HIP_OK(hipMalloc(&d_rec, nrec * TLW * sizeof(unsigned long long)));
+  HIP_OK(hipMemset(d_rec, 0, nrec * TLW * sizeof(unsigned long long)));
+  hipDeviceptr_t sym;
+  size_t sym_bytes = 0;
+  if (hipModuleGetGlobal(&sym, &sym_bytes, (hipModule_t)(uintptr_t)module, "kcg_timeline_ptr") != hipSuccess || sym_bytes != sizeof(void*)) {
+    fprintf(stderr, "this kernel carries no time stamps (only the direct-staging kernel does)\n");
+    return 2;
+  }
+  HIP_OK(hipMemcpy((void*)sym, &d_rec, sizeof(void*), hipMemcpyHostToDevice));
+  const int warm = 300, launches = 100;
+  for (int i = 0; i < warm; ++i) kcg_launch(function, info.grid, info.block, info.lds_bytes, 0, dA, dB, dC);
+  hipEvent_t e0, e1;
+  HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+  HIP_OK(hipEventRecord(e0, 0));
+  for (int i = 0; i < launches; ++i) kcg_launch(function, info.grid, info.block, info.lds_bytes, 0, dA, dB, dC);
+  HIP_OK(hipEventRecord(e1, 0));
+  HIP_OK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  const double period_us = ms * 1e3 / launches;
+  std::vector<unsigned long long> h(nrec * TLW);
+  HIP_OK(hipMemcpy(h.data(), d_rec, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+  HIP_OK(hipFree(d_rec));
+
+  unsigned long long t0 = ~0ull;
+  for (size_t r = 0; r < nrec; ++r) if (h[r * TLW] && h[r * TLW] < t0) t0 = h[r * TLW];
+  struct Stat { double mn = 1e30, mx = -1e30, sum = 0; long n = 0; void add(double v) { mn = v < mn ? v : mn; mx = v > mx ? v : mx; sum += v; ++n; } double mean() const { return n ? sum / n : 0; } };
+  const char* names[5] = {"block_start", "first_tile_landed", "k_loop_done", "stores_issued", "stores_acknowledged"};
+  Stat all[5], xcd_loop[8], xcd_tail[8], xcd_end[8], clk, barrier;
+  for (size_t r = 0; r < nrec; ++r) {
+    const unsigned long long* w = &h[r * TLW];
+    if (!w[0]) continue;
+    for (int p = 0; p < 5; ++p) all[p].add((double)(w[p] - t0) * 0.01);            // 100 MHz -> us
+    const int xcd = (int)((w[6] >> 32) & 0xF) % 8;
+    const double loop_us = (double)(w[2] - w[1]) * 0.01;
+    xcd_loop[xcd].add(loop_us);
+    xcd_tail[xcd].add((double)(w[4] - w[2]) * 0.01);
+    xcd_end[xcd].add((double)(w[4] - t0) * 0.01);
+    if (loop_us > 0) clk.add((double)w[5] / loop_us);                               // cycles per us = MHz
+    if (level >= 2 && w[5]) barrier.add(100.0 * (double)w[7] / (double)w[5]);
+  }
+  printf("{\"timeline\": {\"kernel\": \"%s\", \"level\": %d, \"launch_period_us\": %.2f, \"tflops\": %.1f, \"waves\": %ld,\n", info.kernel_name, level,
+         period_us, flops / (period_us * 1e-6) / 1e12, all[0].n);
+  printf("  \"us_after_first_block_start\": {");
+  for (int p = 0; p < 5; ++p) printf("%s\"%s\": {\"first\": %.2f, \"mean\": %.2f, \"last\": %.2f}", p ? ", " : "", names[p], all[p].mn, all[p].mean(), all[p].mx);
+  printf("},\n  \"gap_to_next_launch_us\": %.2f,\n", period_us - all[4].mx);
+  printf("  \"k_loop_shader_clock_mhz\": {\"min\": %.0f, \"mean\": %.0f, \"max\": %.0f},\n", clk.mn, clk.mean(), clk.mx);
+  if (level >= 2) printf("  \"barrier_wait_pct_of_k_loop_cycles\": {\"min\": %.2f, \"mean\": %.2f, \"max\": %.2f},\n", barrier.mn, barrier.mean(), barrier.mx);
+  printf("  \"by_xcd\": [");
+  for (int x = 0; x < 8; ++x)
+    printf("%s{\"xcd\": %d, \"waves\": %ld, \"k_loop_us_mean\": %.2f, \"k_loop_us_max\": %.2f, \"k_loop_end_to_store_ack_us_mean\": %.2f, \"last_ack_us\": %.2f}",
+           x ? ",\n             " : "", x, xcd_loop[x].n, xcd_loop[x].mean(), xcd_loop[x].mx, xcd_tail[x].mean(), xcd_end[x].mx);
+  printf("]}}\n");
+  return 0;
 }
 
 // minimal reader for the flat {"KEY": int, ...} objects of the tuning files
@@ -310,7 +413,8 @@ int main(int argc, char** argv) {
   memset(&cfg, 0, sizeof(cfg));
   kcg_kernel_info info;
   memset(&info, 0, sizeof(info));
-  int iters = 20, kind = KCG_KIND_AUTO, index = 0, compile_only = 0;
+  int iters = 20, kind = KCG_KIND_AUTO, index = 0, compile_only = 0, timeline = 0;
+  bool normal_dist = false;
   float tol = 0.01f;   // the reference runner's tolerance (runkernel.cpp:34)
   int M = 0, N = 0, K = 0, dt = KCG_DT_FLOAT32, dtc = KCG_DT_FLOAT32, atrans = 1;
 
@@ -326,12 +430,19 @@ int main(int argc, char** argv) {
       else if (!strcmp(argv[i], "--iters")) iters = atoi(argv[i + 1]);
       else if (!strcmp(argv[i], "--tol")) tol = (float)atof(argv[i + 1]);
       else if (!strcmp(argv[i], "--compile-only")) compile_only = atoi(argv[i + 1]);
+      else if (!strcmp(argv[i], "--timeline")) timeline = atoi(argv[i + 1]);
+      else if (!strcmp(argv[i], "--dist")) normal_dist = !strcmp(argv[i + 1], "normal");
       else if (!strcmp(argv[i], "--kind"))
         kind = !strcmp(argv[i + 1], "simt") ? KCG_KIND_SIMT : !strcmp(argv[i + 1], "mfma") ? KCG_KIND_MFMA : KCG_KIND_AUTO;
     }
     if (!read_config(path, index, &cfg)) {
       fprintf(stderr, "cannot read config %d of %s\n", index, path.c_str());
       return 2;
+    }
+    if (timeline > 0) {
+      const char* old = getenv("KCG_EXTRA_FLAGS");
+      std::string flags = std::string(old ? old : "") + " -DKCG_TIMELINE=" + std::to_string(timeline);
+      setenv("KCG_EXTRA_FLAGS", flags.c_str(), 1);
     }
     if (kcg_compile_matmul(&cfg, "gfx950", kind, &info) != KCG_OK) {
       fprintf(stderr, "compile failed: %s\n", kcg_last_error());
@@ -366,8 +477,8 @@ int main(int argc, char** argv) {
   // inputs: logical A[M,K], laid out as the kernel expects
   uint64_t seed = 0x4B4347;
   std::vector<float> a((size_t)M * K), b((size_t)K * N), abuf((size_t)M * K);
-  for (auto& x : a) x = lcg_uniform(seed);
-  for (auto& x : b) x = lcg_uniform(seed);
+  for (auto& x : a) x = normal_dist ? lcg_normal(seed, 0.5f) : lcg_uniform(seed);
+  for (auto& x : b) x = normal_dist ? lcg_normal(seed, 0.5f) : lcg_uniform(seed);
   if (atrans) {
     for (int i = 0; i < M; ++i)
       for (int k = 0; k < K; ++k) abuf[(size_t)k * M + i] = a[(size_t)i * K + k];
@@ -425,6 +536,11 @@ int main(int argc, char** argv) {
   }
   printf("time cost: %.4f ms (median of %d), min %.4f ms;  tflops = %.2f\n", med, iters, mn,
          2.0 * M * N * K / (med * 1e-3) / 1e12);
+  if (timeline > 0) {
+    const int rc = timeline_report(module, function, info, info.block[0] / 64, (uint64_t)dA, (uint64_t)dB, (uint64_t)dC,
+                                   2.0 * M * N * K, timeline);
+    if (rc) return rc;
+  }
   kcg_unload(module);
   return bad ? 1 : 0;
 }

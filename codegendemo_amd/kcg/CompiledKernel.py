@@ -42,6 +42,12 @@ class CompiledKernel:
         if self.m_launcher is not None:
             self.m_launcher.launchKernel(self.device, *args)
 
+    def run_batched(self, a, b, c, batch, stride_a, stride_b, stride_c, alpha=1.0, beta=0.0):
+        """Launch a kernel compiled in the batched-strided form (KCGCompiler(epilogue=...)): problem z of the
+        batch uses the buffers z * stride_* elements further on; alpha and beta take effect in a kernel with
+        the alpha-beta epilogue."""
+        self.m_launcher.launchKernelBatched(self.device, a, b, c, batch, stride_a, stride_b, stride_c, alpha, beta)
+
     def benchmark(self, a, b, c, warmup=1, iters=20, reps=0):
         """HIP-event timing in C: (median_ms, min_ms) per launch."""
         return self.m_launcher.benchmarkKernel(self.device, a, b, c, warmup, iters, reps)

@@ -3,7 +3,6 @@ from enum import Enum
 
 from .CompiledKernel import CompiledKernel
 from .Operators.matmul import KernelArgMatmul, getMatmulSignature
-from .Utils import sizeof
 
 
 class EnumOperator(Enum):
@@ -33,19 +32,23 @@ class UserInputs:
         return self.m_blockDims
 
     def sharedMem(self):
-        """Dynamic LDS bytes for the launch.  The compile result knows what the chosen kernel family
-        needs; without it, the reference's formula (CompiledKernelFactory.py:30-44)."""
+        """Dynamic LDS bytes for the launch: what the kernel inside the code object needs, as the engine
+        reported it at compile time (m_ldsBytes).  A driver written for the reference builds UserInputs from
+        (path, name, config) alone (KCGTask.py:293-296) and relies on the reference's formula
+        (CompiledKernelFactory.py:30-44) here; that formula does not describe this engine's kernels (padded
+        rows in the scalar kernel, fp32 partial sums for 16-bit split-U, static LDS in the direct-staging
+        kernel), so the engine is asked instead: the compile is a cache hit that returns the figure that
+        belongs to exactly this code object.  A code object the engine would not produce for this config
+        (another kernel family was forced) is refused rather than launched with a guessed size."""
         if self.m_ldsBytes is not None:
             return int(self.m_ldsBytes)
-        kp = self.kernelParam
-        sizeAB = kp.BLOCK_SIZE_M * kp.BLOCK_SIZE_K * sizeof(kp.dtype('A')) \
-            + kp.BLOCK_SIZE_N * kp.BLOCK_SIZE_K * sizeof(kp.dtype('B'))
-        if kp.SHARED_PREFETCH > 0:
-            sizeAB *= 2
-        sizeC = -1
-        if kp.LOCAL_SPLIT_U > 1:
-            sizeC = kp.BLOCK_SIZE_M * kp.BLOCK_SIZE_N * kp.LOCAL_SPLIT_U * sizeof(kp.dtype('A'))
-        return max(sizeAB, sizeC)
+        from .. import _native
+        info = _native.compile_matmul(self.kernelParam.values())
+        if info["code_path"] != self.hsacoPath or info["kernel_name"] != self.kernelFuncName:
+            raise ValueError("UserInputs.sharedMem(): the LDS size of this code object is unknown (it is not what "
+                             "the engine builds for this config by default); set m_ldsBytes from the compile result")
+        self.m_ldsBytes = info["lds_bytes"]
+        return int(self.m_ldsBytes)
 
     def numCTA(self):
         n = 1

@@ -27,16 +27,17 @@ class HIPLauncher:
     def _function(self):
         return HIPLoaderST().loadBinary(self.m_kernelLib).m_function
 
-    def _check_operands(self, args):
+    def _check_operands(self, args, batch=1, strides=(0, 0, 0)):
         """A buffer smaller than what the kernel will touch would be a memory fault on the device: refuse it
         on the host.  Only objects that say how large they are (tensors) can be checked."""
         if len(args) != 3:
             raise TypeError(f"GEMM kernel takes 3 device buffers (a, b, c), got {len(args)}")
         if self._need is None:
             return
-        for label, x, need in zip("abc", args, self._need):
+        for label, x, need, stride in zip("abc", args, self._need, strides):
             if hasattr(x, "numel") and hasattr(x, "element_size"):
                 have = int(x.numel()) * int(x.element_size())
+                need = need + (int(batch) - 1) * int(stride) * int(x.element_size())
                 if have < need:
                     raise ValueError(f"operand {label}: {have} bytes, but {self.m_kernelLib.m_kernelFuncName[:60]}... "
                                      f"accesses {need} bytes")
@@ -44,11 +45,23 @@ class HIPLauncher:
                     raise ValueError(f"operand {label} must be contiguous")
 
     def launchKernel(self, devId: int, *args):
+        if self.m_kernelLib.m_kernelFuncName.endswith(("EX_", "EXab_")):
+            raise TypeError("a kernel in the batched-strided form takes strides, alpha and beta: use run_batched")
         self._check_operands(args)
         fn = self._function()
         a, b, c = (_device_address(x) for x in args)
         _native.launch(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,
                        DeviceInfo.get_cuda_stream(devId), a, b, c)
+
+    def launchKernelBatched(self, devId: int, a, b, c, batch, stride_a, stride_b, stride_c, alpha=1.0, beta=0.0):
+        if not self.m_kernelLib.m_kernelFuncName.endswith(("EX_", "EXab_")):
+            raise TypeError("this kernel was not compiled in the batched-strided form (KCGCompiler(epilogue=...))")
+        if batch > 0:
+            self._check_operands((a, b, c), batch, (stride_a, stride_b, stride_c))
+        fn = self._function()
+        a, b, c = (_device_address(x) for x in (a, b, c))
+        _native.launch_batched(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,
+                               DeviceInfo.get_cuda_stream(devId), a, b, c, batch, stride_a, stride_b, stride_c, alpha, beta)
 
     def benchmarkKernel(self, devId: int, a, b, c, warmup=1, iters=20, reps=0):
         """The timing loop of PerfTester in C (kcg_benchmark): (median_ms, min_ms) per launch."""

@@ -113,9 +113,9 @@ int kcg_reference_lds_bytes(const kcg_matmul_cfg* cfg);
 
 /* Block swizzle of Rewriter::BlockMapping (Rewriter.cc:726-761): linear block id -> (by, bx).
  * With xcd_remap != 0 the id is first passed through the engine's XCD remap (hardware block ids are
- * dealt round-robin to the 8 XCDs of an MI355X; the remap gives each XCD one contiguous eighth of
- * the swizzled order so neighbouring tiles share that XCD's L2); applied only when the block count
- * is a multiple of 8.  The kernels are built with the remap unless KCG_XCD_REMAP=0 is set. */
+ * dealt round-robin to the XCDs — 8 on an MI355X, or $KCG_NUM_XCDS — and the remap gives each XCD one
+ * contiguous part of the swizzled order so neighbouring tiles share that XCD's L2); applied only when the
+ * block count is a multiple of the XCD count.  The kernels are built with the remap unless KCG_XCD_REMAP=0. */
 int kcg_block_mapping(const kcg_matmul_cfg* cfg, int bid, int xcd_remap, int32_t* by, int32_t* bx);
 
 /* ---- compile: replaces compile_kernel_matmul (src/main.cc:315-357) -------------------------- */
@@ -131,6 +131,29 @@ int kcg_block_mapping(const kcg_matmul_cfg* cfg, int bid, int xcd_remap, int32_t
  * (that kernel cannot tolerate spills) silently gets the register-staged kernel instead; a
  * "<name>.<hash>.spills" marker in the cache directory remembers the decision. */
 int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch, int kind, kcg_kernel_info* out);
+
+/* ---- batched / strided GEMM with an alpha-beta epilogue ---------------------------------------------
+ * The reference has neither: it lists batched GEMM as the next step of its roadmap (结果汇总.md:21-22) and
+ * profiles its kernels against the vendor sgemm, whose call carries alpha, beta and leading dimensions
+ * (runRoc.cpp:27-28,53-66).  These two entry points give the engine that call shape. */
+enum kcg_epilogue {
+  KCG_EPILOGUE_NONE = 0,       /* C = A B                                   (alpha, beta ignored)   */
+  KCG_EPILOGUE_ALPHA_BETA = 1  /* C = alpha * (A B) + beta * C; beta == 0: C is not read (as in BLAS) */
+};
+
+/* Like kcg_compile_matmul, but the kernel takes (A, B, C, stride_a, stride_b, stride_c, alpha, beta) and
+ * computes problem z of a batch on grid row z from the buffers z * stride_* elements further on.  Same
+ * template, same tuning config, same cache; the kernel symbol is the reference name followed by "EX_"
+ * (no epilogue) or "EXab_" (alpha-beta epilogue).  Launch it with kcg_launch_batched only. */
+int kcg_compile_matmul_ex(const kcg_matmul_cfg* cfg, const char* arch, int kind, int epilogue, kcg_kernel_info* out);
+
+/* Launches `batch` problems of a kernel built by kcg_compile_matmul_ex: grid = {info.grid[0], batch, 1}.
+ * stride_* are in elements of the respective buffer; stride_a or stride_b may be 0 (one operand shared by
+ * the whole batch), stride_c may not (unless batch == 1).  batch <= 65535; batch == 0 launches nothing.
+ * alpha and beta are read only by a kernel with KCG_EPILOGUE_ALPHA_BETA.  Asynchronous on `stream`. */
+int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes,
+                       uint64_t stream, uint64_t a, uint64_t b, uint64_t c, int32_t batch,
+                       int64_t stride_a, int64_t stride_b, int64_t stride_c, float alpha, float beta);
 
 /* The HIP source text that kcg_compile_matmul would hand to hiprtc for this config (the generated
  * instantiation stub; the template header is embedded in the library).  Returns bytes needed. */

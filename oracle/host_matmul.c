@@ -13,9 +13,9 @@
  * Pinning (see tests/test_oracle.py): every function below is checked against closed forms
  * (identity, all-ones, one-hot probes, small-integer matrices that are exact in fp32), against a
  * brute-force pure-Python triple loop on tiny shapes and against numpy float64 matmul.  The reference
- * ships no golden vectors for this path, and its own translation unit (matmul.cpp) does not compile
- * with this toolchain (template-parameter shadowing errors), so there is no build of hostMatmul
- * itself to compare with; see oracle/Makefile.
+ * ships no golden vectors for this path.  Where the reference tree is present, oracle/Makefile also builds
+ * the reference's own hostMatmul (oracle/_ref/libhostmatmul_ref.so) and the tests require bit equality
+ * with oracle_host_matmul_f32_ijk.
  *
  * Built with -ffp-contract=off so that a*b+c is never fused: each C element is the fp32 sum, in
  * ascending k, of individually rounded fp32 products, exactly what the reference loop computes when
@@ -101,6 +101,42 @@ void oracle_matmul_f64(const double* a, const double* b, double* c, int M, int N
       const double av = a_trans ? a[(size_t)k * M + i] : a[(size_t)i * K + k];
       const double* brow = b + (size_t)k * N;
       for (int j = 0; j < N; j++) crow[j] = crow[j] + av * brow[j];
+    }
+  }
+}
+
+/* Batched / strided GEMM with the alpha-beta epilogue of the vendor sgemm call the reference profiles against
+ * (runRoc.cpp:27-28,53-66; batched GEMM is the next item of the reference's roadmap, 结果汇总.md:21-22):
+ *   for z in [0, batch):  C_z = alpha * (A_z B_z) + beta * C_z
+ * with X_z = x + z * stride_x (strides in elements; stride_a / stride_b may be 0).  The product is the same
+ * sequential-k fp32 sum as above; then one multiplication by alpha, one by beta and one addition, each rounded
+ * to fp32.  beta == 0: C is not read (BLAS rule), the result is alpha * (A B).  c is read and overwritten. */
+void oracle_matmul_f32_batched_ab(const float* a, const float* b, float* c, int M, int N, int K, int a_trans, int batch,
+                                  long stride_a, long stride_b, long stride_c, float alpha, float beta, int nthreads) {
+#ifdef _OPENMP
+  if (nthreads <= 0) nthreads = omp_get_max_threads();
+#endif
+  for (int z = 0; z < batch; z++) {
+    const float* az = a + (size_t)z * stride_a;
+    const float* bz = b + (size_t)z * stride_b;
+    float* cz = c + (size_t)z * stride_c;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 4) num_threads(nthreads)
+#endif
+    for (int i = 0; i < M; i++) {
+      float* acc = (float*)malloc((size_t)N * sizeof(float));
+      row_ikj_f32(az, bz, acc, i, M, N, K, a_trans);
+      float* crow = cz + (size_t)i * N;
+      for (int j = 0; j < N; j++) {
+        const float scaled = alpha * acc[j];
+        if (beta == 0.0f) {
+          crow[j] = scaled;
+        } else {
+          const float old = beta * crow[j];
+          crow[j] = scaled + old;
+        }
+      }
+      free(acc);
     }
   }
 }

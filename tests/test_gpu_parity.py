@@ -362,6 +362,30 @@ def test_config5_fp16_4096(oracle):
         assert np.abs(lhs - rhs).max() <= 2e-2 * scale * np.sqrt(M)
 
 
+def test_config5_bf16_4096(oracle):
+    """The config-5 workload with bfloat16 inputs (DATATYPE 3): normal(0, 0.5) rounded to bf16, fp32
+    accumulate/output, the tuned kernel bench.py launches; the oracle runs on the upcast values.
+    Bar: <= 2e-2 relative (to the RMS magnitude of C), plus the column-sum identity over the whole output."""
+    M = N = K = 4096
+    a = quantize(SI.normal((M, K), SI.STREAM_A, std=0.5), 3)
+    b = quantize(SI.normal((K, N), SI.STREAM_B, std=0.5), 3)
+    rows = (2048, 2112)
+    want = oracle.matmul(a, b, a_trans=False, rows=rows)
+    scale = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    cfg = dict(_tuned("gemm_4096_fp16.json"))
+    cfg["DATATYPE_A"] = cfg["DATATYPE_B"] = 3
+    print("[case] config5 with bf16 inputs, tuned kernel", flush=True)
+    got, info = run_gemm(cfg, a, b, MFMA)
+    assert info["lds_bytes"] == 0          # the direct-staging kernel
+    assert not np.isnan(got).any()
+    err = float(np.abs(got[rows[0]:rows[1]] - want).max())
+    print(f"        panel max|err|={err:.3e} scale={scale:.3e} rel={err / scale:.3e}", flush=True)
+    assert err / scale <= 2e-2
+    lhs = got.astype(np.float64).sum(axis=0)
+    rhs = a.astype(np.float64).sum(axis=0) @ b.astype(np.float64)
+    assert np.abs(lhs - rhs).max() <= 2e-2 * scale * np.sqrt(M)
+
+
 def _tuned(name):
     import json
     import os

@@ -12,11 +12,16 @@ pytestmark = pytest.mark.gpu
 
 M = N = K = 512
 CONFIG = make_config(M, N, K, BM=64, BN=64, BK=16, TM=4, TN=4, is_atrans=0)   # precompiled by the build step
+# the direct-staging kernel (static LDS stages, bare barriers and hand-counted waits in its K loop)
+CONFIG_DIRECT = make_config(M, N, K, BM=128, BN=128, BK=32, TM=8, TN=8, is_atrans=0, shared_prefetch=1, reg_prefetch=1)
+CONFIGS = {"register-staged": CONFIG, "direct-staging": CONFIG_DIRECT}
 
 
-def test_launch_is_ordered_on_a_side_stream(oracle):
+@pytest.mark.parametrize("which", list(CONFIGS))
+def test_launch_is_ordered_on_a_side_stream(oracle, which):
     import torch
-    kpm, ui, kernel, info = build_kernel(CONFIG)
+    kpm, ui, kernel, info = build_kernel(CONFIGS[which])
+    assert (info["lds_bytes"] == 0) == (which == "direct-staging")
     a = SI.small_ints((M, K), SI.STREAM_A)
     b = SI.small_ints((K, N), SI.STREAM_B)
     want = oracle.matmul(a, b, a_trans=False)
@@ -26,7 +31,7 @@ def test_launch_is_ordered_on_a_side_stream(oracle):
     a_dev = torch.empty((M, K), dtype=torch.float32, device="cuda:0")
     c_dev = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda:0")
     torch.cuda.synchronize()
-    print("[case] side-stream launch 512^3", flush=True)
+    print(f"[case] side-stream launch 512^3 {which}", flush=True)
     with torch.cuda.stream(side):
         # upload -> GEMM -> scale, all queued on the side stream without host synchronisation:
         # the GEMM must see the uploaded A and the scaling must see the finished C
@@ -39,19 +44,20 @@ def test_launch_is_ordered_on_a_side_stream(oracle):
     assert np.array_equal(got, 2.0 * want)
 
 
-def test_launch_can_be_captured_in_a_hip_graph(oracle):
+@pytest.mark.parametrize("which", list(CONFIGS))
+def test_launch_can_be_captured_in_a_hip_graph(oracle, which):
     """A launch through the boundary allocates nothing and synchronises nothing, so a caller may capture it
     into a HIP graph (once the module is loaded: the first run of a kernel loads it, which is not capturable).
     The graph is replayed four times on different operands with eager work and synchronisations in between;
     every replay must equal the eager result and the oracle bit for bit (small integers)."""
     import torch
-    kpm, ui, kernel, info = build_kernel(CONFIG)
+    kpm, ui, kernel, info = build_kernel(CONFIGS[which])
     b = SI.small_ints((K, N), SI.STREAM_B)
     b_dev = to_device(b, torch.float32)
     a_dev = torch.zeros((M, K), dtype=torch.float32, device="cuda:0")
     c_dev = torch.zeros((M, N), dtype=torch.float32, device="cuda:0")
     c_eager = torch.zeros((M, N), dtype=torch.float32, device="cuda:0")
-    print("[case] graph capture 512^3", flush=True)
+    print(f"[case] graph capture 512^3 {which}", flush=True)
     kernel.run(a_dev, b_dev, c_dev)      # loads the module
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()

@@ -81,7 +81,21 @@ def test_compiler_return_shape_and_factory(tmp_path, monkeypatch):
     assert (gx, gy, gz, bx, by, bz) == (256, 1, 1, 256, 1, 1)
     assert KCGCompiler().compile_kernel_matmul(*kpm.values()) == res
     ui = UserInputs(path, name, kpm)
-    assert ui.sharedMem() == 2 * (64 + 64) * 16 * 4       # reference formula when the engine value is unknown
+    # a reference-style driver never sets m_ldsBytes (KCGTask.py:293-296): the engine is asked, not the formula
+    assert ui.m_ldsBytes is None
+    comp = KCGCompiler()
+    comp.compileKernel(kpm)
+    assert ui.sharedMem() == comp.lastInfo["lds_bytes"] == 2 * (64 + 64) * 16 * 4
+    # where formula and kernel disagree (row padding of the scalar kernel for A[M,K]) the engine's figure wins
+    kpm0 = kernelArgFromConfig(make_config(1024, 1024, 1024, shared_prefetch=1, is_atrans=0))
+    comp.kind = 1
+    p0, n0 = comp.compileKernel(kpm0)[0][:2]
+    forced = UserInputs(p0, n0, kpm0)
+    with pytest.raises(ValueError):
+        forced.sharedMem()              # not the default family for this config: unknown, refused
+    comp.kind = 0
+    p1, n1 = comp.compileKernel(kpm0)[0][:2]
+    assert UserInputs(p1, n1, kpm0).sharedMem() == comp.lastInfo["lds_bytes"]
     ui.m_gridDims, ui.m_blockDims = [gx, gy, gz], [bx, by, bz]
     assert ui.numCTA() == 256 and ui.operatorKind == EnumOperator.Matmul
     kernel = CompiledKernelFactory.getKernel(ui, 0)

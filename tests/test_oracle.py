@@ -129,3 +129,80 @@ def test_linearity_and_f64_gemm(oracle):
     bd = SI.uniform((K, N), 75).astype(np.float64)
     assert np.allclose(oracle.matmul_f64(ad, bd, 0), ad @ bd, rtol=0, atol=1e-13 * K)
     assert np.array_equal(oracle.matmul_f64(np.ascontiguousarray(ad.T), bd, 1), oracle.matmul_f64(ad, bd, 0))
+
+
+def test_reference_build_of_hostMatmul_is_bit_equal():
+    """oracle/_ref: the reference's own hostMatmul, compiled from matmul.cpp:2349-2360 where it lies, against the
+    restatement: the reference's single-config test tile (test.py:32-57) and two seeded shapes."""
+    from tests import oracle_binding
+    ref = oracle_binding.load_reference_build()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built (no reference tree on this machine)")
+    orc = oracle_binding.load()
+    for (M, N, K), seeds in (((64, 48, 32), (81, 82)), ((96, 200, 257), (83, 84)), ((33, 17, 1000), (85, 86))):
+        a = SI.normal((M, K), seeds[0])
+        b = SI.normal((K, N), seeds[1])
+        a_km = SI.a_operand(a, 1)
+        want = ref(a_km, b)
+        assert np.array_equal(orc.ijk(a_km, b, 1), want)
+        assert np.array_equal(orc.matmul(a_km, b, 1), want)
+        assert np.array_equal(orc.matmul(a, b, 0), want)          # the row-major layout of the same product
+
+
+# ---- batched / strided GEMM with the alpha-beta epilogue: pinned by what the mathematics fixes -----------
+def _batched_inputs(M, N, K, batch, ints=True):
+    gen = (lambda shp, st: SI.small_ints(shp, st)) if ints else (lambda shp, st: SI.normal(shp, st))
+    a = np.stack([gen((M, K), 100 + z) for z in range(batch)])
+    b = np.stack([gen((K, N), 200 + z) for z in range(batch)])
+    c0 = np.stack([gen((M, N), 300 + z) for z in range(batch)])
+    return a, b, c0
+
+
+@pytest.mark.parametrize("a_trans", [0, 1])
+def test_batched_ab_alpha1_beta0_is_the_plain_product_per_slice(oracle, a_trans):
+    M, N, K, batch = 24, 40, 56, 3
+    a, b, c0 = _batched_inputs(M, N, K, batch, ints=False)
+    a_buf = np.stack([SI.a_operand(a[z], a_trans) for z in range(batch)])
+    c0[:] = np.nan                                   # beta == 0: C must not be read
+    got = oracle.batched_ab(a_buf, b, c0, M, N, K, a_trans, batch, (M * K, K * N, M * N), 1.0, 0.0).reshape(batch, M, N)
+    for z in range(batch):
+        assert np.array_equal(got[z], oracle.matmul(a_buf[z], b[z], a_trans))
+
+
+def test_batched_ab_strides(oracle):
+    """Padding between the problems of a batch and a B shared by the whole batch (stride 0)."""
+    M, N, K, batch = 8, 16, 24, 4
+    a, b, c0 = _batched_inputs(M, N, K, batch)
+    sa, sc = M * K + 5, M * N + 3
+    a_flat = np.full(batch * sa, np.nan, np.float32)
+    c_flat = np.full(batch * sc, -7.0, np.float32)
+    for z in range(batch):
+        a_flat[z * sa:z * sa + M * K] = a[z].ravel()
+    got = oracle.batched_ab(a_flat, b[0], c_flat, M, N, K, 0, batch, (sa, 0, sc), 1.0, 0.0)
+    for z in range(batch):
+        assert np.array_equal(got[z * sc:z * sc + M * N].reshape(M, N), oracle.matmul(a[z], b[0], 0))
+        assert (got[z * sc + M * N:(z + 1) * sc] == -7.0).all()          # the padding is not touched
+
+
+def test_batched_ab_beta_and_alpha_exact_on_integers(oracle):
+    M, N, K, batch = 16, 24, 32, 2
+    a, b, c0 = _batched_inputs(M, N, K, batch)
+    strides = (M * K, K * N, M * N)
+    prod = np.stack([(a[z].astype(np.int64) @ b[z].astype(np.int64)) for z in range(batch)])
+    for alpha, beta in ((1.0, 1.0), (2.0, -3.0), (-0.5, 0.25), (0.0, 1.0), (3.0, 0.0)):
+        got = oracle.batched_ab(a, b, c0, M, N, K, 0, batch, strides, alpha, beta).reshape(batch, M, N)
+        want = alpha * prod.astype(np.float64) + beta * c0.astype(np.float64)        # exact in fp64 and in fp32
+        assert np.array_equal(got.astype(np.float64), want), (alpha, beta)
+
+
+def test_batched_ab_linearity_in_alpha_on_powers_of_two(oracle):
+    """Scaling by a power of two commutes with fp32 rounding: result(alpha = 2^p) = 2^p * result(alpha = 1)."""
+    M, N, K = 12, 20, 300
+    a, b, c0 = _batched_inputs(M, N, K, 1, ints=False)
+    strides = (M * K, K * N, M * N)
+    base = oracle.batched_ab(a, b, c0, M, N, K, 0, 1, strides, 1.0, 0.0)
+    for p in (-3, 1, 5):
+        assert np.array_equal(oracle.batched_ab(a, b, c0, M, N, K, 0, 1, strides, 2.0 ** p, 0.0), base * np.float32(2.0 ** p))
+    # and beta = 1 adds C0 once, rounded once
+    got = oracle.batched_ab(a, b, c0, M, N, K, 0, 1, strides, 1.0, 1.0)
+    assert np.array_equal(got, (base + c0.ravel()).astype(np.float32))

@@ -139,3 +139,24 @@ def test_best_perf_bookkeeping():
     back.parseFromJson(j["results"][0])
     assert back.acc == 3.0 and back.kpm == rs[1].kpm
     PerfTester.BestPerf = []
+
+
+def test_stored_library_time_is_keyed_by_shape_types_and_device(workdir):
+    """The library GEMM time kept in _cache/benchmarkTorchEps.log is reused only for the shape, types and
+    device it was measured for (a tuning file with mixed shapes must not inherit the first shape's time)."""
+    os.makedirs(PathManager.default_cache_dir(), exist_ok=True)
+    old_shape, old_eps = PerfTester._shape, PerfTester.torch_eps
+    try:
+        PerfTester._shape = (1024, 1024, 1024, 4, 4)
+        with open(PerfTester._torchEpsStoreFile(), "w") as f:
+            json.dump({"key": PerfTester._torch_eps_key(), "ms": 0.04}, f)
+        PerfTester.torch_eps = 0.0
+        assert PerfTester._read_torch_eps_from_file() and PerfTester.torch_eps == 0.04
+        PerfTester._shape = (2048, 2048, 2048, 4, 4)
+        PerfTester.torch_eps = 0.0
+        assert not PerfTester._read_torch_eps_from_file() and PerfTester.torch_eps == 0.0
+        with open(PerfTester._torchEpsStoreFile(), "w") as f:
+            f.write("0.123")                                       # the reference's bare number: ignored
+        assert not PerfTester._read_torch_eps_from_file()
+    finally:
+        PerfTester._shape, PerfTester.torch_eps = old_shape, old_eps
