@@ -10,7 +10,11 @@ uniform[-1,1) inputs already resident in HBM).  The JSON line printed at the end
   value / ms_per_step : whole-job throughput over exactly K steps between two device synchronisations
   roofline            : 2MNK / (average launch duration measured with HIP events on the launch
                         stream over the same K launches) against the fp32 MFMA peak of MI355X
-  fp16                : the same two figures for the fp16-input / fp32-accumulate kernel at 4096^3
+  roofline_steady     : the same kernel after 100 untimed launches, HIP-event average over 200 launches (the
+                        part's clocks need several milliseconds under load to settle; with a short warm-up that
+                        ramp lies inside the K timed steps)
+  fp16, bf16          : the same figures for the 16-bit-input / fp32-accumulate kernels at 4096^3, each checked
+                        against the oracle on a row panel
   cpu_baseline        : the CPU oracle (a port of the reference's hostMatmul arithmetic) timed on this
                         box's host cores on a bounded row panel of the same product
 
@@ -68,7 +72,9 @@ def build_kernel(config):
     ui.m_gridDims, ui.m_blockDims = [gx, gy, gz], [bx, by, bz]
     ui.m_ldsBytes = comp.lastInfo["lds_bytes"]
     ui.operatorKind = EnumOperator.Matmul
-    return kpm, CompiledKernelFactory.getKernel(ui, 0), comp.lastInfo
+    kernel = CompiledKernelFactory.getKernel(ui, 0)
+    kernel.n_regs           # loads the code object now (otherwise the first launch would)
+    return kpm, kernel, comp.lastInfo
 
 
 def make_inputs(kpm, dist):
@@ -279,13 +285,29 @@ def main():
                           "tflops": fl / (ms_launch16 * 1e-3) / 1e12}))
         return
 
+    # ---- preparation: every kernel built and loaded, every operand resident in HBM, before anything is timed.
+    # The timed legs below then follow each other without host work in between (input generation takes
+    # seconds, during which an idle GPU drops its clocks again).
     cfg32 = load_tuned(args.fp32_config or "gemm_4096_fp32.json")
     kpm, kernel, info = build_kernel(cfg32)
     a, b, A, B, C = make_inputs(kpm, "uniform")
-    ms_step, ms_launch = time_steps(kernel, A, B, C, args.steps, args.warmup)
     flops = 2.0 * kpm.M * kpm.N * kpm.K
+    legs16 = []           # (key, label, kpm, kernel, info, A, B, C)
+    if not args.no_fp16:
+        cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
+        cfgb = dict(cfg16)
+        cfgb["DATATYPE_A"] = cfgb["DATATYPE_B"] = 3      # the same config with bfloat16 inputs
+        for key, label, cfg in (("fp16", "f16", cfg16), ("bf16", "bf16", cfgb)):
+            k_, kern_, info_ = build_kernel(cfg)
+            _, _, A_, B_, C_ = make_inputs(k_, "normal")
+            legs16.append((key, label, k_, kern_, info_, A_, B_, C_))
+    torch.cuda.synchronize()
+
+    # ---- timed legs
+    ms_step, ms_launch = time_steps(kernel, A, B, C, args.steps, args.warmup)
     value = flops / (ms_step * 1e-3) / 1e12
     achieved = flops / (ms_launch * 1e-3) / 1e12
+    steady32 = steady_roofline(kernel, A, B, C, flops, PEAK_TFLOPS["f32"])
     c_host = C.cpu().numpy()
     traffic32, traffic32_note = measured_traffic(info["kernel_name"])
     lib_ms = time_library_gemm(A, B, kpm.isATranspose, args.steps, args.warmup)
@@ -305,63 +327,45 @@ def main():
                      "frac": achieved / PEAK_TFLOPS["f32"], "traffic": traffic32, "traffic_source": traffic32_note,
                      "launch_ms": ms_launch,
                      "hbm_gbs_algorithmic": (4.0 * (kpm.M * kpm.K + kpm.K * kpm.N + kpm.M * kpm.N)) / (ms_launch * 1e-3) / 1e9},
+        "roofline_steady": steady32,
     }
-    out["roofline_steady"] = steady_roofline(kernel, A, B, C, flops, PEAK_TFLOPS["f32"])
-
     out["library_gemm"] = {"source": "torch.matmul (rocBLAS/hipBLASLt) on the same buffers, same timing loop",
                            "f32_tflops": flops / (lib_ms * 1e-3) / 1e12}
-    if not args.no_fp16:
-        cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
-        kpm16, kernel16, info16 = build_kernel(cfg16)
-        _, _, A16, B16, C16 = make_inputs(kpm16, "normal")
-        ms_step16, ms_launch16 = time_steps(kernel16, A16, B16, C16, args.steps, args.warmup)
-        ach16 = flops / (ms_launch16 * 1e-3) / 1e12
-        traffic16, traffic16_note = measured_traffic(info16["kernel_name"])
-        lib16_ms = time_library_gemm(A16, B16, kpm16.isATranspose, args.steps, args.warmup)
-        out["library_gemm"]["f16_tflops"] = flops / (lib16_ms * 1e-3) / 1e12
-        out["library_gemm"]["f16_note"] = "torch.matmul on fp16 operands returns fp16: the library writes 32 MiB of C, this engine 64 MiB of fp32"
-        out["fp16"] = {"value": flops / (ms_step16 * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_step16,
-                       "dtype": "f16 in, f32 accumulate/out", "kernel": info16["kernel_name"],
-                       "roofline": {"bound": "mfma", "achieved": ach16, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
-                                    "frac": ach16 / PEAK_TFLOPS["f16"], "traffic": traffic16, "traffic_source": traffic16_note,
-                                    "launch_ms": ms_launch16},
-                       "roofline_steady": steady_roofline(kernel16, A16, B16, C16, flops, PEAK_TFLOPS["f16"])}
+    for key, label, k_, kern_, info_, A_, B_, C_ in legs16:
+        ms_step_, ms_launch_ = time_steps(kern_, A_, B_, C_, args.steps, args.warmup)
+        ach_ = flops / (ms_launch_ * 1e-3) / 1e12
+        traffic_, traffic_note_ = measured_traffic(info_["kernel_name"])
+        out[key] = {"value": flops / (ms_step_ * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_step_,
+                    "dtype": f"{label} in, f32 accumulate/out", "kernel": info_["kernel_name"],
+                    "roofline": {"bound": "mfma", "achieved": ach_, "peak": PEAK_TFLOPS[label], "unit": "TFLOP/s",
+                                 "frac": ach_ / PEAK_TFLOPS[label], "traffic": traffic_, "traffic_source": traffic_note_,
+                                 "launch_ms": ms_launch_},
+                    "roofline_steady": steady_roofline(kern_, A_, B_, C_, flops, PEAK_TFLOPS[label])}
+        if key == "fp16":
+            lib16_ms = time_library_gemm(A_, B_, k_.isATranspose, args.steps, args.warmup)
+            out["library_gemm"]["f16_tflops"] = flops / (lib16_ms * 1e-3) / 1e12
+            out["library_gemm"]["f16_note"] = "torch.matmul on fp16 operands returns fp16: the library writes 32 MiB of C, this engine 64 MiB of fp32"
 
-        if not args.no_cpu:     # (skipped in profiling runs, like the CPU leg)
-            # parity of the fp16 result: a 64-row panel against the oracle run on the upcast fp16 values
-            a16h, b16h = make_inputs_host(kpm16)
-            out["fp16"]["parity"] = half_parity(C16, a16h, b16h)
-            if not out["fp16"]["parity"]["ok"]:
+    # ---- checks and side information (nothing below is timed)
+    if not args.no_cpu:     # (skipped in profiling runs, like the CPU leg)
+        for key, label, k_, kern_, info_, A_, B_, C_ in legs16:
+            # a 64-row panel of the result against the oracle run on the upcast 16-bit values
+            ah, bh = make_inputs_host(k_)
+            out[key]["parity"] = half_parity(C_, ah, bh)
+            del ah, bh
+            if not out[key]["parity"]["ok"]:
                 print(json.dumps(out))
-                print("bench.py: fp16 GPU result differs from the oracle beyond tolerance", file=sys.stderr)
+                print(f"bench.py: {key} GPU result differs from the oracle beyond tolerance", file=sys.stderr)
                 sys.exit(1)
-            pc = power_and_clocks(kernel16, A16, B16, C16)
+        if legs16:
+            _, _, _, kern_, _, A_, B_, C_ = legs16[0]
+            pc = power_and_clocks(kern_, A_, B_, C_)
             if pc:
                 out["fp16"]["power_and_clocks"] = pc
             pc = power_and_clocks(kernel, A, B, C)
             if pc:
                 out["roofline"]["power_and_clocks"] = pc
-
-        # the same config with bfloat16 inputs (same kernel template, same data distribution)
-        cfgb = dict(cfg16)
-        cfgb["DATATYPE_A"] = cfgb["DATATYPE_B"] = 3
-        kpmb, kernelb, infob = build_kernel(cfgb)
-        _, _, Ab, Bb, Cb = make_inputs(kpmb, "normal")
-        ms_stepb, ms_launchb = time_steps(kernelb, Ab, Bb, Cb, args.steps, args.warmup)
-        achb = flops / (ms_launchb * 1e-3) / 1e12
-        out["bf16"] = {"value": flops / (ms_stepb * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_stepb,
-                       "dtype": "bf16 in, f32 accumulate/out", "kernel": infob["kernel_name"],
-                       "roofline": {"bound": "mfma", "achieved": achb, "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
-                                    "frac": achb / PEAK_TFLOPS["f16"], "launch_ms": ms_launchb},
-                       "roofline_steady": steady_roofline(kernelb, Ab, Bb, Cb, flops, PEAK_TFLOPS["f16"])}
-        if not args.no_cpu:
-            abh, bbh = make_inputs_host(kpmb)
-            out["bf16"]["parity"] = half_parity(Cb, abh, bbh)
-            if not out["bf16"]["parity"]["ok"]:
-                print(json.dumps(out))
-                print("bench.py: bf16 GPU result differs from the oracle beyond tolerance", file=sys.stderr)
-                sys.exit(1)
-        del Ab, Bb, Cb
+    if legs16:
         # What the matrix pipeline alone sustains on this box (register operands, no memory traffic), on
         # zeros and on data like the workload's: the stand-alone runner measures it in a child process.
         # fp16 GEMMs on this part run at its power limit, so the second figure bounds any fp16 kernel.
@@ -371,6 +375,7 @@ def main():
             p = subprocess.run([runner, "--mfma-peak", "f16"], capture_output=True, text=True, timeout=120)
             if p.returncode == 0:
                 out["fp16"]["mfma_only_sustained"] = json.loads(p.stdout.strip().splitlines()[-1])["mfma_peak"]
+    del legs16
 
     if not args.no_cpu:
         base, panel, rows = cpu_baseline(a, b)

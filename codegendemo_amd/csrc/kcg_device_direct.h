@@ -23,6 +23,26 @@ namespace kcg {
 #ifndef KCG_TIMELINE
 #define KCG_TIMELINE 0
 #endif
+// Diagnostic builds only (never set by the library itself; C is then WRONG): the K loop of the direct-staging
+// kernel without its global->LDS fetches (the stages keep the first tiles, which the prologue still fetches)
+// resp. without its fragment reads (the matrix-core instructions keep running on the first fragments).
+// Timing such builds shows what each part of the data movement costs a launch.
+#ifndef KCG_DIAG_NO_FETCH
+#define KCG_DIAG_NO_FETCH 0
+#endif
+#ifndef KCG_DIAG_NO_LDS_READS
+#define KCG_DIAG_NO_LDS_READS 0
+#endif
+// ... and with every fetch reading K tile 0 again (the fetches stay, but all of them hit in L2: what remains
+// of their cost is the path from L2 into LDS, what disappears is the traffic between L2 and memory)
+#ifndef KCG_DIAG_FETCH_TILE0
+#define KCG_DIAG_FETCH_TILE0 0
+#endif
+// Cache-policy bits of the global->LDS fetch instructions (bit 0: sc0, bit 1: nt, bit 4: sc1).  A block reads
+// every operand byte exactly once, so nothing is gained by keeping the lines in the compute unit's vector cache.
+#ifndef KCG_FETCH_AUX
+#define KCG_FETCH_AUX 0
+#endif
 // 1: the direct-staging kernel writes C with non-temporal stores (C is written once and not read again by
 // the kernel: the stores need not displace operand panels from L2)
 #ifndef KCG_C_NT
@@ -49,7 +69,8 @@ __device__ __forceinline__ unsigned long long tl_cycles() {
 // Family 2b: matrix-core kernel with direct global->LDS staging.
 //
 // Every lane fetches one 16-byte chunk (G = 4 fp32 or 8 fp16/bf16 elements) with
-// global_load_lds_dwordx4; a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
+// global_load_lds_dwordx4 (one 4-byte element with global_load_lds_dword where M, N or K of an fp32 problem is
+// not a multiple of 4, so that rows do not start on 16-byte boundaries); a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
 // ds_write and no vector ALU work is spent on staging, and with NST stages the fetch of a tile can be in
 // flight for NST-1 K tiles.  The LDS image keeps the orientation of global memory:
 //   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/G chunks of G k values each; a fragment
@@ -126,13 +147,18 @@ struct DirectPlan {
   // block tile extents: a power of two, or a multiple of 16 chunks (the bank swizzle of a row-contiguous
   // tile exchanges chunks inside aligned groups of 16, so a row must consist of whole groups): 192, 320, ...
   static constexpr bool tile_ok(int x) { return pow2(x) || (x > 0 && x % (16 * G) == 0); }
+  // What a lane fetches: a whole 16-byte chunk where every row of A and B starts on a 16-byte boundary (M, N and K
+  // multiples of G); otherwise, for 4-byte elements, a single element (the same instruction with a 4-byte payload:
+  // a wave's 64 elements land in 256 consecutive bytes of LDS).  2-byte elements have no such form.
+  static constexpr bool CHUNK_FETCH = C::M % G == 0 && C::N % G == 0 && C::K % G == 0;
+  static constexpr int FG = CHUNK_FETCH ? G : 1;                  // elements per lane and fetch instruction
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
-      // edge tiles in M and N are fine; K needs one full tile (its remainder is a multiple of G like K itself)
+      // edge tiles in M and N are fine; K needs one full tile
       SPW > 0 && C::K >= C::BK && WM / MF >= 2 && tile_ok(C::BM) && tile_ok(C::BN) && pow2(C::BK) && C::BM >= 32 && C::BN >= 32 &&
-      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (C::M % G == 0) &&
-      (C::N % G == 0) && (C::K % G == 0) && 2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
+      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (CHUNK_FETCH || ES == 4) &&
+      2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
       (long)C::BM * C::K * ES < (1L << 31) && (long)C::BK * C::M * ES < (1L << 31) && (long)C::BK * C::N * ES < (1L << 31);
   // LDS stages: as many as fit in 160 KiB (or in half of it, see PAIR below), at most 4 (fetch distance =
@@ -142,7 +168,7 @@ struct DirectPlan {
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
   // and no more than the fetch counter can tell apart: the wait for tile kt+1 allows the fetches of
   // NST-2 younger tiles in flight, and that counter has 6 bits
-  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
+  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / FG) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
   static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
   static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
   // Two blocks on a compute unit beat one block with deeper staging when the launch has more blocks than the
@@ -188,8 +214,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int CHK = BK / G;                           // chunks per row of a k-contiguous tile
   constexpr int NCHA = BM / G, NCHB = BN / G;           // chunks per row of a row-contiguous tile
   constexpr int A_BYTES = BM * BK * ES, B_BYTES = BN * BK * ES, STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int NIA = (BM * BK / G) / (64 * NW);        // fetch instructions per wave and tile, operand A
-  constexpr int NIB = (BN * BK / G) / (64 * NW);
+  constexpr int FG = P::FG, GPC = G / FG;               // elements per lane and fetch; fetch granules per chunk
+  constexpr int NIA = (BM * BK / FG) / (64 * NW);       // fetch instructions per wave and tile, operand A
+  constexpr int NIB = (BN * BK / FG) / (64 * NW);
+  constexpr int FETCH_BYTES = 64 * FG * ES;             // LDS bytes one fetch instruction of a wave fills
   typedef Mfma<T, MF> MI;
   typedef typename MI::Acc Acc;
   typedef typename MI::Frag Frag;
@@ -232,31 +260,36 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // never changes: the K loop spends no vector instruction on addresses.
   // kvalid: how many k rows/values of the tile exist (BK, or KR for the partial tile)
   auto off_a = [&](int idx, int kvalid) -> unsigned {
-    const int s = 64 * (wave * NIA + idx) + lane;     // physical chunk slot inside the A stage
+    const int p = 64 * (wave * NIA + idx) + lane;     // physical fetch-granule slot inside the A stage
+    const int s = p / GPC, e = (p % GPC) * FG;        // chunk slot; first element of the granule inside its chunk
     if constexpr (AK) {
       int row = s / CHK;
       const int cp = s % CHK;
-      int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
-      if (c * G >= kvalid) c = 0;
+      const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
+      int k = c * G + e;
+      if (k >= kvalid) k = 0;
       if constexpr (EDGE_M) row = cmin(row, M - 1 - m0);
-      return (unsigned)((row * K + c * G) * ES);
+      return (unsigned)((row * K + k) * ES);
     } else {
       int k = s / NCHA;
       const int cp = s % NCHA;
-      int c = cp ^ swz_n(k, NCHA);
+      const int c = cp ^ swz_n(k, NCHA);
+      int m = c * G + e;
       if (k >= kvalid) k = 0;
-      if constexpr (EDGE_M) c = cmin(c, (M - m0) / G - 1);
-      return (unsigned)((k * M + c * G) * ES);
+      if constexpr (EDGE_M) m = cmin(m, M - m0 - FG);
+      return (unsigned)((k * M + m) * ES);
     }
   };
   auto off_b = [&](int j, int kvalid) -> unsigned {
-    const int s = 64 * (wave * NIB + j) + lane;
+    const int p = 64 * (wave * NIB + j) + lane;
+    const int s = p / GPC, e = (p % GPC) * FG;
     int k = s / NCHB;
     const int cp = s % NCHB;
-    int c = cp ^ swz_n(k, NCHB);
+    const int c = cp ^ swz_n(k, NCHB);
+    int n = c * G + e;
     if (k >= kvalid) k = 0;
-    if constexpr (EDGE_N) c = cmin(c, (N - n0) / G - 1);
-    return (unsigned)((k * N + c * G) * ES);
+    if constexpr (EDGE_N) n = cmin(n, N - n0 - FG);
+    return (unsigned)((k * N + n) * ES);
   };
   unsigned voff_a[NIA], voff_b[NIB];
 #pragma unroll
@@ -272,6 +305,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // tile offset with vector instructions); kept apart, the fetch uses its scalar-base addressing form.
   struct TileBase { const char* a; const char* b; };
   auto tile_base = [&](int kt) {
+    if constexpr (KCG_DIAG_FETCH_TILE0 != 0) kt = 0;
     TileBase t = {a_base + kt * A_KT_BYTES, b_base + kt * B_KT_BYTES};
     asm("" : "+s"(t.a), "+s"(t.b));
     return t;
@@ -289,7 +323,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       }
       const char* src = tb.a + (unsigned long)off;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + 1024 * (wave * NIA + idx)), 16, 0, 0);
+                                       (__attribute__((address_space(3))) void*)(st + FETCH_BYTES * (wave * NIA + idx)), P::FG * P::ES, 0, KCG_FETCH_AUX);
     } else {
       const int j = idx - NIA;
       unsigned off;
@@ -300,7 +334,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       }
       const char* src = tb.b + (unsigned long)off;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + A_BYTES + 1024 * (wave * NIB + j)), 16, 0, 0);
+                                       (__attribute__((address_space(3))) void*)(st + A_BYTES + FETCH_BYTES * (wave * NIB + j)), P::FG * P::ES, 0, KCG_FETCH_AUX);
     }
   };
   constexpr int NFETCH = NIA + NIB;
@@ -319,7 +353,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragTr {                                    // 16-bit, row-contiguous tile: two transposing 64-bit reads
     u32x2 h[2];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
-    __device__ __forceinline__ void keep_if(bool keep) { h[0] = keep ? h[0] : u32x2{0, 0}; h[1] = keep ? h[1] : u32x2{0, 0}; }
+    // nvalid: how many of the lane's G consecutive k values exist (16-bit: all or none, K being a multiple of G)
+    __device__ __forceinline__ void keep_first(int nvalid) { const bool keep = nvalid > 0; h[0] = keep ? h[0] : u32x2{0, 0}; h[1] = keep ? h[1] : u32x2{0, 0}; }
     __device__ __forceinline__ Frag get() const {
       const u32x4 v = {h[0].x, h[0].y, h[1].x, h[1].y};
       return __builtin_bit_cast(Frag, v);
@@ -328,9 +363,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragS4 {                                    // 32-bit, row-contiguous tile: four 32-bit reads
     unsigned w[4];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3])); }
-    __device__ __forceinline__ void keep_if(bool keep) {
+    __device__ __forceinline__ void keep_first(int nvalid) {      // w[e] is the lane's e-th k value
 #pragma unroll
-      for (int e = 0; e < 4; ++e) w[e] = keep ? w[e] : 0u;
+      for (int e = 0; e < 4; ++e) w[e] = e < nvalid ? w[e] : 0u;
     }
     __device__ __forceinline__ Frag get() const {
       const u32x4 v = {w[0], w[1], w[2], w[3]};
@@ -340,7 +375,13 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragLd {                                    // k-contiguous tile: one 128-bit read
     u32x4 q;
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(q)); }
-    __device__ __forceinline__ void keep_if(bool keep) { q = keep ? q : u32x4{0, 0, 0, 0}; }
+    __device__ __forceinline__ void keep_first(int nvalid) {
+      if constexpr (ES == 4) {                                      // one k value per 32-bit word
+        q.x = 0 < nvalid ? q.x : 0u; q.y = 1 < nvalid ? q.y : 0u; q.z = 2 < nvalid ? q.z : 0u; q.w = 3 < nvalid ? q.w : 0u;
+      } else {
+        q = nvalid > 0 ? q : u32x4{0, 0, 0, 0};                     // 16-bit: all or none (K is a multiple of G)
+      }
+    }
     __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
   };
   typedef typename Select<ES == 2, FragTr, FragS4>::type FragRc;
@@ -491,7 +532,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   FragA fa[TMI];
   FragB fb[2][TNI];
   static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
-  static_for<0, DA>([&](auto i) { load_a(IntC<0>(), IntC<0>(), i, &fa[decltype(i)::value]); });
+  static_for<0, (KCG_DIAG_NO_LDS_READS ? TMI : DA)>([&](auto i) { load_a(IntC<0>(), IntC<0>(), i, &fa[decltype(i)::value]); });
+  if constexpr (KCG_DIAG_NO_LDS_READS != 0 && SPW > 1)
+    static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<1>(), j, &fb[1][decltype(j)::value]); });
   wait_lds();   // the counted waits of the loop assume that nothing older than its own reads is in flight
 
   // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists; HP: the
@@ -512,14 +555,14 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     const TileBase tbn = tile_base(HN ? kt + NST : 0);
     const TileBase tbp = tile_base(HP ? kt - 1 + NST : 0);
     // In the partial K tile a k-step may reach beyond K: every fragment layout of this kernel gives a lane
-    // the G consecutive k values that start at S*KS + G*(lane/MF), so such a lane holds nothing but
-    // k >= K (what was fetched in their place is arbitrary) and clears its fragments.
+    // the G consecutive k values that start at S*KS + G*(lane/MF); those of them that are >= K (what was
+    // fetched in their place is arbitrary) are cleared before use.
     constexpr bool PARTIAL = KR > 0 && NS == SPWT && decltype(has1)::value == false && (KR % KS != 0);
     static_for<0, NS>([&](auto s_c) {
       constexpr int S = decltype(s_c)::value;
       constexpr bool LAST = (S == NS - 1);
       constexpr bool MASK = PARTIAL && LAST;
-      const bool keep = S * KS + G * fgrp < KR;
+      const int nvalid = KR - (S * KS + G * fgrp);   // how many of this lane's G consecutive k values lie below K
       constexpr int PB = (CUR * SPW + S) & 1;       // half of the B double buffer this step computes from
       constexpr bool NEXT = !LAST || H1;            // a next step exists, its fragments are read under this one
       static_for<0, TMI>([&](auto i_c) {
@@ -558,18 +601,19 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         if constexpr (MASK) {
           // (pinned again behind the selects: they must have been issued before the wait state that
           // separates them from the matrix-core instruction reading their results)
-          fa[I].keep_if(keep);
+          fa[I].keep_first(nvalid);
           fa[I].pin();
           if constexpr (I == 0) {
 #pragma unroll
             for (int j = 0; j < TNI; ++j) {
-              fb[PB][j].keep_if(keep);
+              fb[PB][j].keep_first(nvalid);
               fb[PB][j].pin();
             }
           }
           asm volatile("s_nop 1" ::: "memory");
         }
-        if constexpr (I + DA < TMI) load_a(IntC<CUR>(), IntC<S>(), IntC<I + DA>(), &fa[I + DA]);
+        if constexpr (KCG_DIAG_NO_LDS_READS != 0) {
+        } else if constexpr (I + DA < TMI) load_a(IntC<CUR>(), IntC<S>(), IntC<I + DA>(), &fa[I + DA]);
         else if constexpr (!LAST) load_a(IntC<CUR>(), IntC<S + 1>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
         else if constexpr (H1) load_a(IntC<NXT>(), IntC<0>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
         static_for<0, TNI>([&](auto j_c) {
@@ -582,7 +626,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           MI::run_tied(acc[I][JC], fb[PB][JC].get(), fa[I].get());
           static_for<0, TNI>([&](auto jj_c) {
             constexpr int JJ = decltype(jj_c)::value;
-            if constexpr (SP::slot_b(JJ) == I * TNI + J) {
+            if constexpr (KCG_DIAG_NO_LDS_READS == 0 && SP::slot_b(JJ) == I * TNI + J) {
               if constexpr (!LAST) load_b(IntC<CUR>(), IntC<S + 1>(), jj_c, &fb[PB ^ 1][JJ]);
               else if constexpr (H1) load_b(IntC<NXT>(), IntC<0>(), jj_c, &fb[PB ^ 1][JJ]);
             }
@@ -590,8 +634,10 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 #pragma unroll
           for (int f = 0; f < NFETCH; ++f) {
             const int pos = BAR + (f * SPREAD) / NFETCH;          // position on the time line that starts at this tile
-            if (HN && pos == slot) fetch_item(f, tbn, IntC<CUR>(), pn_c);
-            if (HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>(), pp_c);
+            // (diagnostic builds: 1 drops every fetch of the K loop, 2 those of A only, 3 those of B only)
+            const bool fetch_on = KCG_DIAG_NO_FETCH == 0 || (KCG_DIAG_NO_FETCH == 2 && f >= NIA) || (KCG_DIAG_NO_FETCH == 3 && f < NIA);
+            if (fetch_on && HN && pos == slot) fetch_item(f, tbn, IntC<CUR>(), pn_c);
+            if (fetch_on && HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>(), pp_c);
           }
           __builtin_amdgcn_sched_barrier(0);
         });
@@ -658,8 +704,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-        if constexpr (C::EPI) epi_apply<TC, float, 4, (EDGE_M || EDGE_N), true>(v, Cm, row, col, N, M, N, ep);
-        gstore<TC, float, 4, (EDGE_M || EDGE_N), true, (KCG_C_NT != 0)>(Cm, v, row, col, N, M, N);
+        // (N a multiple of 4: every group of four columns is one aligned 16-byte vector, inside or outside as a whole)
+        if constexpr (C::EPI) epi_apply<TC, float, 4, (EDGE_M || EDGE_N), (N % 4 == 0)>(v, Cm, row, col, N, M, N, ep);
+        gstore<TC, float, 4, (EDGE_M || EDGE_N), (N % 4 == 0), (KCG_C_NT != 0)>(Cm, v, row, col, N, M, N);
       }
 #if KCG_TIMELINE
   asm volatile("" ::: "memory");

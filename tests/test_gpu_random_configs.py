@@ -131,6 +131,54 @@ def random_edge_configs(n_matrix=50, n_simt=30, n_direct=25, seed=20250311):
     return out
 
 
+def random_odd_direct_configs(n=30, seed=20251125):
+    """-> [(config, kind)]: a third fixed sample: fp32 configs that take the direct-staging kernel although M, N
+    or K is not a multiple of the 16-byte vector (rows of A and B then do not start on 16-byte boundaries and
+    the kernel fetches element by element): odd extents in every dimension, K remainders of any length, both A
+    layouts, all matrix-core tile shapes and block sizes."""
+    rng = random.Random(seed)
+    out = []
+    while len(out) < n:
+        BM, BN = rng.choice([32, 64, 128, 256]), rng.choice([32, 64, 128, 256])
+        BK = rng.choice([8, 16, 32, 64])
+        kt = rng.choice([1, 2, 3, 4, 5, 7, 9, 12, 17])
+        kw = dict(BM=BM, BN=BN, BK=BK, TM=rng.choice([2, 4, 8, 16]), TN=rng.choice([2, 4, 8, 16]),
+                  warp_layout=rng.choice([(8, 8), (8, 8), (4, 16), (16, 4)]), dtype=4, is_atrans=rng.choice([0, 1]),
+                  block_mapping=rng.choice([0, 2, 4, 8]), shared_prefetch=1, reg_prefetch=1,
+                  M=BM * rng.choice([1, 2]) - rng.choice([0, 1, 2, 3, 5, 7, BM - 1, BM // 2 + 1]),
+                  N=BN * rng.choice([1, 2, 3]) - rng.choice([0, 1, 2, 3, 6, 9, BN - 1, BN // 2 - 1]),
+                  K=BK * kt + rng.choice([0, 1, 2, 3, 5, 6, 7, 9, 13, 31]) % BK)
+        if kw["M"] <= 0 or kw["N"] <= 0 or (kw["M"] % 4 == 0 and kw["N"] % 4 == 0 and kw["K"] % 4 == 0):
+            continue
+        try:
+            cfg = make_config(**kw)
+            v = kernelArgFromConfig(cfg).values()
+            if _native.is_valid_config(v, _native.KIND_MFMA) and \
+                    "DIRECT = true" in _native.instantiation_source(v, _native.KIND_MFMA):
+                out.append((cfg, _native.KIND_MFMA))
+        except (ValueError, _native.KcgError):
+            continue
+    return out
+
+
+def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
+    cases = random_odd_direct_configs()
+    direct = 0
+    for i, (cfg, kind) in enumerate(cases):
+        M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+        a = SI.small_ints((M, K), SI.STREAM_A, lim=2)
+        b = SI.small_ints((K, N), SI.STREAM_B, lim=2)
+        print(f"[case] random odd direct {i} {kernelArgFromConfig(cfg).values()}", flush=True)
+        got, info = run_gemm(cfg, a, b, kind)
+        direct += int(info["lds_bytes"] == 0)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        bad = int((got.astype(np.float64) != want).sum()) + int(np.isnan(got).sum())
+        assert bad == 0, f"random odd config {i} ({info['kernel_name']}): {bad} wrong elements"
+    # (a few of the sample need more registers for their per-lane fetch offsets than they have and are built with
+    # register staging instead: the library's rule for direct-staging builds that would spill)
+    assert direct >= 20
+
+
 def test_random_edge_config_sample_is_bit_exact():
     """Entries in {-1, 0, 1}: every sum is an integer of magnitude <= K, exact in fp32 and, for the 16-bit
     outputs (K <= 255 there), in fp16 and bf16 as well."""
