@@ -172,10 +172,12 @@ def test_instantiation_source_carries_the_config():
 @pytest.mark.parametrize("shape,kw,direct", [
     ((4096, 1536, 1000), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # K = 62*16 + 8: one k-step of 8 left over
     ((4096, 1536, 1004), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # remainder 12: a whole k-step and half of one
-    ((4096, 1536, 1002), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),     # K is not a multiple of the 16-byte vector
+    ((4096, 1536, 1002), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # fp32, K not a multiple of the 16-byte vector: element-granular fetch
+    ((4095, 1533, 1001), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # fp32, odd in every dimension
     ((4096, 1536, 8), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),        # not even one full K tile
     ((200, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),         # rows and columns beyond M and N
-    ((202, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),        # M is not a multiple of the 16-byte vector
+    ((202, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),         # fp32, M not a multiple of the 16-byte vector
+    ((256, 252, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=3, dtype_c=4), False),  # bf16, N % 8 != 0: no element-granular form
     ((256, 256, 992), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),    # 16x16x32 tiles: k-steps of 32
     ((256, 256, 1008), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # remainder 48 = 1.5 k-steps
     ((256, 256, 1004), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), False),  # K % 8 != 0
