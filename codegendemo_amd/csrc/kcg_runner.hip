@@ -6,12 +6,14 @@
 // print, naive `gemm_kernel` + `verify_kernel`, matmul.cpp:2327-2348,2386-2553).
 //
 //   kcg_runner --config <file.json> [--index i] [--kind auto|simt|mfma] [--iters n] [--tol t]
-//              [--dist uniform|normal] [--timeline 1|2]
+//              [--dist uniform|normal] [--timeline 1|2] [--dump-c file]
 //       compiles entry i of a {"cfgs": [...]} file (or a single flat config object) through
 //       libkcg_gemm.so, loads it, verifies it against the naive kernel and times it
 //       (--compile-only 1 stops after the compile: fills the code-object cache on a host without a GPU).
 //       --dist: operands uniform on [-1,1) (default) or normal(0, 0.5), the distribution the 16-bit
 //       benchmark uses (on a power-limited part the speed of a matrix-core kernel depends on the data).
+//       --dump-c: writes the kernel's C (raw fp32, row-major) so that it can be checked outside this program; the
+//       inputs are a pure function of the shape: a 64-bit LCG (seed 0x4B4347) fills A[M,K] then B[K,N] in row-major order.
 //       --timeline: builds the direct-staging kernel with its in-kernel time stamps (-DKCG_TIMELINE=level
 //       added to $KCG_EXTRA_FLAGS), runs it back to back and prints where the time of one launch goes:
 //       block start, first K tile landed, K loop done, C stores issued / acknowledged, per XCD and over
@@ -415,6 +417,7 @@ int main(int argc, char** argv) {
   memset(&info, 0, sizeof(info));
   int iters = 20, kind = KCG_KIND_AUTO, index = 0, compile_only = 0, timeline = 0;
   bool normal_dist = false;
+  const char* dump_c = nullptr;
   float tol = 0.01f;   // the reference runner's tolerance (runkernel.cpp:34)
   int M = 0, N = 0, K = 0, dt = KCG_DT_FLOAT32, dtc = KCG_DT_FLOAT32, atrans = 1;
 
@@ -432,6 +435,7 @@ int main(int argc, char** argv) {
       else if (!strcmp(argv[i], "--compile-only")) compile_only = atoi(argv[i + 1]);
       else if (!strcmp(argv[i], "--timeline")) timeline = atoi(argv[i + 1]);
       else if (!strcmp(argv[i], "--dist")) normal_dist = !strcmp(argv[i + 1], "normal");
+      else if (!strcmp(argv[i], "--dump-c")) dump_c = argv[i + 1];
       else if (!strcmp(argv[i], "--kind"))
         kind = !strcmp(argv[i + 1], "simt") ? KCG_KIND_SIMT : !strcmp(argv[i + 1], "mfma") ? KCG_KIND_MFMA : KCG_KIND_AUTO;
     }
@@ -527,6 +531,17 @@ int main(int argc, char** argv) {
   memcpy(&maxerr, &maxbits, 4);
   if (bad) printf("have %llu error! first at (y=%llu, x=%llu), max |err| %.3e (tol %.3g)\n", bad, first / N, first % N, maxerr, tol);
   else printf("no error! max |err| %.3e (tol %.3g)\n", maxerr, tol);
+
+  if (dump_c) {   // the kernel's result as raw fp32, row-major [M, N]: lets a caller check it against its own reference
+    std::vector<float> hc((size_t)M * N);
+    HIP_OK(hipMemcpy(hc.data(), dC, hc.size() * sizeof(float), hipMemcpyDeviceToHost));
+    FILE* f = fopen(dump_c, "wb");
+    if (!f || fwrite(hc.data(), sizeof(float), hc.size(), f) != hc.size()) {
+      fprintf(stderr, "cannot write %s\n", dump_c);
+      return 3;
+    }
+    fclose(f);
+  }
 
   float med = 0.f, mn = 0.f;
   if (kcg_benchmark(function, info.grid, info.block, info.lds_bytes, 0, (uint64_t)dA, (uint64_t)dB, (uint64_t)dC, 20, iters, 0,

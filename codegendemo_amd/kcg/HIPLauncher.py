@@ -58,6 +58,10 @@ class HIPLauncher:
             raise TypeError("this kernel was not compiled in the batched-strided form (KCGCompiler(epilogue=...))")
         if batch > 0:
             self._check_operands((a, b, c), batch, (stride_a, stride_b, stride_c))
+            # every problem's buffers must be as aligned as the first one's: the kernels move 16-byte vectors
+            for label, x, stride in zip("abc", (a, b, c), (stride_a, stride_b, stride_c)):
+                if batch > 1 and hasattr(x, "element_size") and (int(stride) * int(x.element_size())) % 16:
+                    raise ValueError(f"stride_{label} = {stride} elements is not a multiple of 16 bytes")
         fn = self._function()
         a, b, c = (_device_address(x) for x in (a, b, c))
         _native.launch_batched(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,

@@ -173,7 +173,8 @@ int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int 
 int kcg_launch(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes,
                uint64_t stream, uint64_t a, uint64_t b, uint64_t c);
 
-/* The timing loop of PerfTester._test_perf (KCGTask.py:162-181) done in C with HIP events on
+/* (For kernels built by kcg_compile_matmul only: it launches with the three-pointer argument list.)
+ * The timing loop of PerfTester._test_perf (KCGTask.py:162-181) done in C with HIP events on
  * `stream`: `warmup` untimed launches, then `iters` samples; each sample brackets `reps` back-to-back
  * launches (reps <= 0: chosen so one sample lasts >= 1 ms) and is divided by reps.
  * Outputs per-launch median and minimum in milliseconds. */

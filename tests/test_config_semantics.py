@@ -98,6 +98,24 @@ def test_block_mapping_is_a_permutation(M, N, BM, BN, G, xcd):
     assert seen == set(itertools.product(range(gy), range(gx)))
 
 
+@pytest.mark.parametrize("nx", [1, 2, 4, 8])
+def test_xcd_remap_follows_the_partition_description(nx, monkeypatch):
+    """$KCG_NUM_XCDS describes the partition the kernels are built for (8 on an MI355X in single-partition mode):
+    the remap stays a permutation, gives every XCD one contiguous part of the swizzled order, and the count
+    reaches the instantiation stub together with the compute-unit count."""
+    monkeypatch.setenv("KCG_NUM_XCDS", str(nx))
+    monkeypatch.setenv("KCG_NUM_CUS", str(32 * nx))
+    cfg = make_config(1024, 1024, 64, BM=64, BN=64, block_mapping=8)      # 256 blocks
+    v = vals(cfg)
+    plain = [_native.block_mapping(v, b, False) for b in range(256)]
+    remapped = [_native.block_mapping(v, b, True) for b in range(256)]
+    assert sorted(remapped) == sorted(plain)
+    for hw in range(256):                    # hardware id hw runs on XCD hw % nx and takes position ... of that XCD's part
+        assert remapped[hw] == plain[(hw % nx) * (256 // nx) + hw // nx]
+    src = _native.instantiation_source(v, _native.KIND_MFMA)
+    assert f"NUM_XCD = {nx};" in src and f"NUM_CU = {32 * nx};" in src
+
+
 def test_block_mapping_formula():
     """Rewriter.cc:726-761 (isCol=true): G = BLOCK_MAPPING, H = N/BN;
     by = (bid / (G*H))*G + bid % G, bx = (bid % (G*H)) / G when (M/BM) % G == 0, identity otherwise."""

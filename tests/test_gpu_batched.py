@@ -158,6 +158,8 @@ def test_launch_batched_argument_checks():
         kernel.run_batched(a, b, c, 70000, 0, 0, 0)
     with pytest.raises(ValueError):
         kernel.run_batched(a, b, c, 3, 128 * 64, 64 * 192, 128 * 192)      # buffers hold two problems, not three
+    with pytest.raises(ValueError):
+        kernel.run_batched(a, b, c, 2, 128 * 64 - 2, 64 * 192, 128 * 192)  # second problem's A not 16-byte aligned
     with pytest.raises(TypeError):
         kernel.run(a, b, c)                                                # the three-pointer launch does not fit this kernel
     kernel.run_batched(a, b, c, 0, 0, 0, 0)                                # empty batch: nothing launched
