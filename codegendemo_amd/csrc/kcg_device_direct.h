@@ -69,8 +69,8 @@ __device__ __forceinline__ unsigned long long tl_cycles() {
 // Family 2b: matrix-core kernel with direct global->LDS staging.
 //
 // Every lane fetches one 16-byte chunk (G = 4 fp32 or 8 fp16/bf16 elements) with
-// global_load_lds_dwordx4 (one 4-byte element with global_load_lds_dword where M, N or K of an fp32 problem is
-// not a multiple of 4, so that rows do not start on 16-byte boundaries); a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
+// global_load_lds_dwordx4 (4 bytes with global_load_lds_dword where M, N or K is not a multiple of G, so that rows do
+// not start on 16-byte boundaries: one fp32 element, or two 16-bit ones when M, N and K are even); a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
 // ds_write and no vector ALU work is spent on staging, and with NST stages the fetch of a tile can be in
 // flight for NST-1 K tiles.  The LDS image keeps the orientation of global memory:
 //   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/G chunks of G k values each; a fragment
@@ -148,16 +148,18 @@ struct DirectPlan {
   // tile exchanges chunks inside aligned groups of 16, so a row must consist of whole groups): 192, 320, ...
   static constexpr bool tile_ok(int x) { return pow2(x) || (x > 0 && x % (16 * G) == 0); }
   // What a lane fetches: a whole 16-byte chunk where every row of A and B starts on a 16-byte boundary (M, N and K
-  // multiples of G); otherwise, for 4-byte elements, a single element (the same instruction with a 4-byte payload:
-  // a wave's 64 elements land in 256 consecutive bytes of LDS).  2-byte elements have no such form.
+  // multiples of G); otherwise 4 bytes (the same instruction with a 4-byte payload: a wave's 64 pieces land in 256
+  // consecutive bytes of LDS) — one 4-byte element, or two 2-byte elements where M, N and K are even.
   static constexpr bool CHUNK_FETCH = C::M % G == 0 && C::N % G == 0 && C::K % G == 0;
-  static constexpr int FG = CHUNK_FETCH ? G : 1;                  // elements per lane and fetch instruction
+  static constexpr int FGMIN = ES <= 4 ? 4 / ES : 1;              // elements in 4 bytes
+  static constexpr bool PIECE_FETCH = ES <= 4 && C::M % FGMIN == 0 && C::N % FGMIN == 0 && C::K % FGMIN == 0;
+  static constexpr int FG = CHUNK_FETCH ? G : FGMIN;              // elements per lane and fetch instruction
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
       // edge tiles in M and N are fine; K needs one full tile
       SPW > 0 && C::K >= C::BK && WM / MF >= 2 && tile_ok(C::BM) && tile_ok(C::BN) && pow2(C::BK) && C::BM >= 32 && C::BN >= 32 &&
-      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (CHUNK_FETCH || ES == 4) &&
+      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (CHUNK_FETCH || PIECE_FETCH) &&
       2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
       (long)C::BM * C::K * ES < (1L << 31) && (long)C::BK * C::M * ES < (1L << 31) && (long)C::BK * C::N * ES < (1L << 31);
@@ -353,8 +355,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   struct FragTr {                                    // 16-bit, row-contiguous tile: two transposing 64-bit reads
     u32x2 h[2];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
-    // nvalid: how many of the lane's G consecutive k values exist (16-bit: all or none, K being a multiple of G)
-    __device__ __forceinline__ void keep_first(int nvalid) { const bool keep = nvalid > 0; h[0] = keep ? h[0] : u32x2{0, 0}; h[1] = keep ? h[1] : u32x2{0, 0}; }
+    // nvalid: how many of the lane's G = 8 consecutive k values exist (an even number: K is even).  h[0] holds
+    // k values 0..3 of them (two per 32-bit word), h[1] the values 4..7.
+    __device__ __forceinline__ void keep_first(int nvalid) {
+      h[0].x = 0 < nvalid ? h[0].x : 0u; h[0].y = 2 < nvalid ? h[0].y : 0u;
+      h[1].x = 4 < nvalid ? h[1].x : 0u; h[1].y = 6 < nvalid ? h[1].y : 0u;
+    }
     __device__ __forceinline__ Frag get() const {
       const u32x4 v = {h[0].x, h[0].y, h[1].x, h[1].y};
       return __builtin_bit_cast(Frag, v);
@@ -378,8 +384,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     __device__ __forceinline__ void keep_first(int nvalid) {
       if constexpr (ES == 4) {                                      // one k value per 32-bit word
         q.x = 0 < nvalid ? q.x : 0u; q.y = 1 < nvalid ? q.y : 0u; q.z = 2 < nvalid ? q.z : 0u; q.w = 3 < nvalid ? q.w : 0u;
-      } else {
-        q = nvalid > 0 ? q : u32x4{0, 0, 0, 0};                     // 16-bit: all or none (K is a multiple of G)
+      } else {                                                      // two k values per 32-bit word, K is even
+        q.x = 0 < nvalid ? q.x : 0u; q.y = 2 < nvalid ? q.y : 0u; q.z = 4 < nvalid ? q.z : 0u; q.w = 6 < nvalid ? q.w : 0u;
       }
     }
     __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }

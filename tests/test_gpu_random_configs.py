@@ -161,13 +161,45 @@ def random_odd_direct_configs(n=30, seed=20251125):
     return out
 
 
+def random_even_16bit_direct_configs(n=20, seed=20251126):
+    """-> [(config, kind)]: fp16 / bf16 configs that take the direct-staging kernel although M, N or K is not a
+    multiple of 8 (all three even: the kernel then fetches two elements per lane), K remainders of any even length,
+    both A layouts, 16-bit and fp32 outputs."""
+    rng = random.Random(seed)
+    out = []
+    while len(out) < n:
+        dtype = rng.choice([2, 3])
+        BM, BN = rng.choice([32, 64, 128, 256]), rng.choice([32, 64, 128, 256])
+        BK = rng.choice([16, 32, 64])
+        out16 = rng.random() < 0.3
+        kt = rng.choice([1, 2, 3] if out16 else [1, 2, 3, 4, 5, 7, 9, 12])
+        kw = dict(BM=BM, BN=BN, BK=BK, TM=rng.choice([2, 4, 8, 16]), TN=rng.choice([2, 4, 8, 16]),
+                  warp_layout=rng.choice([(8, 8), (8, 8), (4, 16), (16, 4)]), dtype=dtype, dtype_c=dtype if out16 else 4,
+                  is_atrans=rng.choice([0, 1]), block_mapping=rng.choice([0, 2, 4, 8]), shared_prefetch=1, reg_prefetch=1,
+                  M=BM * rng.choice([1, 2]) - rng.choice([0, 2, 4, 6, 10, BM - 2, BM // 2 + 2]),
+                  N=BN * rng.choice([1, 2, 3]) - rng.choice([0, 2, 4, 6, 12, BN - 2, BN // 2 - 2]),
+                  K=BK * kt + rng.choice([0, 2, 4, 6, 10, 14, 30]) % BK)
+        if kw["M"] <= 0 or kw["N"] <= 0 or (kw["M"] % 8 == 0 and kw["N"] % 8 == 0 and kw["K"] % 8 == 0):
+            continue
+        try:
+            cfg = make_config(**kw)
+            v = kernelArgFromConfig(cfg).values()
+            if _native.is_valid_config(v, _native.KIND_MFMA) and \
+                    "DIRECT = true" in _native.instantiation_source(v, _native.KIND_MFMA):
+                out.append((cfg, _native.KIND_MFMA))
+        except (ValueError, _native.KcgError):
+            continue
+    return out
+
+
 def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
-    cases = random_odd_direct_configs()
+    cases = random_odd_direct_configs() + random_even_16bit_direct_configs()
     direct = 0
     for i, (cfg, kind) in enumerate(cases):
         M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
-        a = SI.small_ints((M, K), SI.STREAM_A, lim=2)
-        b = SI.small_ints((K, N), SI.STREAM_B, lim=2)
+        lim = 2 if cfg["DATATYPE_C"] == 4 else 1       # 16-bit outputs: |sums| <= K <= 222 stay exact
+        a = SI.small_ints((M, K), SI.STREAM_A, lim=lim)
+        b = SI.small_ints((K, N), SI.STREAM_B, lim=lim)
         print(f"[case] random odd direct {i} {kernelArgFromConfig(cfg).values()}", flush=True)
         got, info = run_gemm(cfg, a, b, kind)
         direct += int(info["lds_bytes"] == 0)
@@ -176,7 +208,7 @@ def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
         assert bad == 0, f"random odd config {i} ({info['kernel_name']}): {bad} wrong elements"
     # (a few of the sample need more registers for their per-lane fetch offsets than they have and are built with
     # register staging instead: the library's rule for direct-staging builds that would spill)
-    assert direct >= 20
+    assert direct >= 35
 
 
 def test_random_edge_config_sample_is_bit_exact():
