@@ -33,6 +33,9 @@ namespace kcg {
 #ifndef KCG_DIAG_NO_LDS_READS
 #define KCG_DIAG_NO_LDS_READS 0
 #endif
+// -DKCG_DIAG_EVEN_XCD_SLEEP=n (C stays correct): the blocks on even-numbered XCDs sleep n * 64 cycles in front of every
+// K-tile barrier.  On a power-limited kernel the odd-numbered XCDs then run faster by about what the even ones lose:
+// the XCDs share one power budget.
 // ... and with every fetch reading K tile 0 again (the fetches stay, but all of them hit in L2: what remains
 // of their cost is the path from L2 into LDS, what disappears is the traffic between L2 and memory)
 #ifndef KCG_DIAG_FETCH_TILE0
@@ -233,6 +236,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   int by, bx;
   block_coords<C>(blockIdx.x, by, bx);
   const int m0 = by * BM, n0 = bx * BN;
+#if defined(KCG_DIAG_EVEN_XCD_SLEEP)
+  const bool even_xcd = (__builtin_amdgcn_s_getreg(20 | (31 << 11)) & 1) == 0;
+#endif
 #if KCG_TIMELINE
   unsigned long long tl[KCG_TL_WORDS] = {};
   tl[0] = tl_realtime();
@@ -591,6 +597,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           // flight (vmcnt(0)), which would expose the whole memory latency at each tile.  What has
           // to be complete at this point is exactly what the two waits above ask for.
           asm volatile("" ::: "memory");
+#if defined(KCG_DIAG_EVEN_XCD_SLEEP)
+          if (even_xcd) __builtin_amdgcn_s_sleep(KCG_DIAG_EVEN_XCD_SLEEP);
+#endif
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
 #if KCG_TIMELINE >= 2
