@@ -168,7 +168,7 @@ def time_library_gemm(A, B, a_trans, steps, warmup):
     return ev0.elapsed_time(ev1) / steps
 
 
-def cpu_baseline(a, b, ijk_seconds=8.0):
+def cpu_baseline(a, b, ijk_seconds=5.0):
     """Times the CPU oracle on this box's host cores: the threaded loop over the WHOLE 4096^3 product
     (best of 3; it is also the parity reference for the GPU result) and, for the record, the
     reference's own loop order (i-j-k, one thread) on a row panel sized to a few seconds."""
@@ -193,15 +193,28 @@ def cpu_baseline(a, b, ijk_seconds=8.0):
     probe = time.perf_counter() - t0
     rows_ijk = int(max(1, min(64, ijk_seconds / max(probe, 1e-4))))
     t0 = time.perf_counter()
-    orc.ijk(a, b, 0, rows=(0, rows_ijk))
+    panel_ijk = orc.ijk(a, b, 0, rows=(0, rows_ijk))
     dt_ijk = time.perf_counter() - t0
-    return {
+    out = {
         "value": 2.0 * M * N * K / best / 1e12, "unit": "TFLOPS", "cores": threads, "kind": "port",
         "sample": f"whole fp32 4096^3 product on the same inputs, best of 3 runs ({best:.2f} s each), "
                   f"i-k-j loop order, OpenMP over rows",
         "reference_loop_order": {"value": 2.0 * rows_ijk * N * K / dt_ijk / 1e12, "unit": "TFLOPS", "cores": 1,
                                  "sample": f"i-j-k order (hostMatmul), first {rows_ijk} rows of C, {dt_ijk:.1f} s"},
-    }, full, M
+    }
+    # the reference's own hostMatmul (matmul.cpp:2349-2360, built by oracle/Makefile where the reference tree was
+    # present) on the same row panel: it wants A stored [K, M], so the panel's rows go in as a [K, rows] operand
+    ref = oracle_binding.load_reference_build()
+    if ref is not None:
+        import numpy as np
+        a_km = np.ascontiguousarray(a[:rows_ijk].T)
+        t0 = time.perf_counter()
+        got = ref(a_km, b)
+        dt_ref = time.perf_counter() - t0
+        out["reference_build"] = {"value": 2.0 * rows_ijk * N * K / dt_ref / 1e12, "unit": "TFLOPS", "cores": 1, "kind": "reference",
+                                  "sample": f"the reference's hostMatmul compiled from its own source, first {rows_ijk} rows of C, {dt_ref:.1f} s",
+                                  "bit_equal_to_port": bool(np.array_equal(got, panel_ijk))}
+    return out, full, M
 
 
 def power_and_clocks(kernel, A, B, C, seconds=2.0):
