@@ -33,14 +33,14 @@ namespace kcg {
 #ifndef KCG_DIAG_NO_LDS_READS
 #define KCG_DIAG_NO_LDS_READS 0
 #endif
-// -DKCG_DIAG_EVEN_XCD_SLEEP=n (C stays correct): the blocks on even-numbered XCDs sleep n * 64 cycles in front of every
-// K-tile barrier.  On a power-limited kernel the odd-numbered XCDs then run faster by about what the even ones lose:
-// the XCDs share one power budget.
 // ... and with every fetch reading K tile 0 again (the fetches stay, but all of them hit in L2: what remains
 // of their cost is the path from L2 into LDS, what disappears is the traffic between L2 and memory)
 #ifndef KCG_DIAG_FETCH_TILE0
 #define KCG_DIAG_FETCH_TILE0 0
 #endif
+// -DKCG_DIAG_EVEN_XCD_SLEEP=n (C stays correct): the blocks on even-numbered XCDs sleep n * 64 cycles in front of every
+// K-tile barrier.  On a power-limited kernel the odd-numbered XCDs then run faster by about what the even ones lose:
+// the XCDs share one power budget.
 // Cache-policy bits of the global->LDS fetch instructions (bit 0: sc0, bit 1: nt, bit 4: sc1).  A block reads
 // every operand byte exactly once, so nothing is gained by keeping the lines in the compute unit's vector cache.
 #ifndef KCG_FETCH_AUX

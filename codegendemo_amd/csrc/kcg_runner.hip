@@ -31,7 +31,8 @@
 //   kcg_runner --launch-cost
 //       the fixed costs a short GEMM pays per launch on this GPU: the period of back-to-back launches of
 //       an empty kernel (1 block; 256 blocks; 256 blocks with 64 KiB of LDS each) and of a kernel that
-//       only writes 64 MiB (the fp32 result of a 4096 x 4096 product)
+//       only writes 64 MiB (the fp32 result of a 4096 x 4096 product); and, on a line of its own before that,
+//       when a global->LDS fetch issued behind 32 stores of the same wave lands and when the wave's counter says so
 //
 // Build: make -C codegendemo_amd/csrc runner      (hipcc --offload-arch=gfx950)
 #include <hip/hip_runtime.h>
@@ -255,6 +256,64 @@ __global__ __launch_bounds__(256) void write_tiles(float* __restrict__ out) {
     }
 }
 
+// What a wave can know about a global->LDS fetch it issued behind its own stores.  Every wave (one per block, one
+// block per compute unit) optionally issues NSTORES 16-byte-per-lane stores to cold lines, then one 16-byte-per-lane
+// fetch of cache-resident data into LDS that it had filled with a marker, and measures (shader-clock cycles)
+//   [0] until the fetched data is visible in LDS (polling the last lane's slot),
+//   [1] until s_waitcnt vmcnt(0) returns (the wave's only counter for fetches and stores alike).
+template <int NSTORES>
+__global__ __launch_bounds__(64) void fetch_behind_stores(const float4* __restrict__ src, float4* __restrict__ sink,
+                                                            unsigned long long* __restrict__ out) {
+  __shared__ __attribute__((aligned(1024))) float4 lds[64];
+  const int lane = threadIdx.x;
+  lds[lane] = float4{-1.f, -1.f, -1.f, -1.f};
+  __syncthreads();
+  // every store instruction writes 16 rows x 64 bytes, rows 1 KiB apart (the shape of the GEMM epilogue's stores)
+  float4* mine = sink + ((size_t)blockIdx.x * 512 + lane % 16) * 64 + lane / 16;
+  const float4 v = {1.f, 2.f, 3.f, 4.f};
+  const unsigned lds_probe = (unsigned)(unsigned long)lds + 63 * 16;
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime();
+#pragma unroll
+  for (int i = 0; i < NSTORES; ++i) mine[(size_t)i * 16 * 64] = v;
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + lane),
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+  unsigned long long t_seen = 0;
+  for (int spin = 0; spin < 200000; ++spin) {                        // bounded: every wave leaves the loop
+    // (read with an instruction the compiler does not connect with the fetch: it would wait for vmcnt(0) first)
+    unsigned probe;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(probe) : "v"(lds_probe) : "memory");
+    if (__builtin_amdgcn_readfirstlane((int)probe) != __float_as_int(-1.f)) {
+      t_seen = __builtin_amdgcn_s_memtime();
+      break;
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);                                // vmcnt(0), nothing else
+  const unsigned long long t_cnt = __builtin_amdgcn_s_memtime();
+  if (lane == 0) {
+    out[blockIdx.x * 2] = t_seen ? t_seen - t0 : 0;
+    out[blockIdx.x * 2 + 1] = t_cnt - t0;
+  }
+}
+
+template <int NSTORES>
+static void run_fetch_behind_stores(double* seen_cycles, double* counted_cycles) {
+  float4 *src, *sink;
+  unsigned long long* out;
+  HIP_OK(hipMalloc(&src, 64 * sizeof(float4)));
+  HIP_OK(hipMalloc(&sink, (size_t)256 * 512 * 64 * sizeof(float4)));   // 128 MiB
+  HIP_OK(hipMalloc(&out, 512 * sizeof(unsigned long long)));
+  HIP_OK(hipMemset(src, 0, 64 * sizeof(float4)));                    // zeros differ from the marker
+  for (int i = 0; i < 20; ++i) hipLaunchKernelGGL((fetch_behind_stores<NSTORES>), dim3(256), dim3(64), 0, 0, src, sink, out);
+  HIP_OK(hipDeviceSynchronize());
+  unsigned long long h[512];
+  HIP_OK(hipMemcpy(h, out, sizeof(h), hipMemcpyDeviceToHost));
+  double a = 0, b = 0;
+  for (int i = 0; i < 256; ++i) { a += (double)h[2 * i]; b += (double)h[2 * i + 1]; }
+  *seen_cycles = a / 256;
+  *counted_cycles = b / 256;
+  HIP_OK(hipFree(src)); HIP_OK(hipFree(sink)); HIP_OK(hipFree(out));
+}
+
 template <class F>
 static double launch_period_us(F launch, int n) {
   for (int i = 0; i < 200; ++i) launch();
@@ -283,6 +342,12 @@ static int launch_cost_main() {
   const double t128 = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<128, false>), dim3(256), dim3(256), 0, 0, sink); }, 500);
   const double t64nt = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<64, true>), dim3(256), dim3(256), 0, 0, sink); }, 500);
   const double t128nt = launch_period_us([&] { hipLaunchKernelGGL((write_tiles<128, true>), dim3(256), dim3(256), 0, 0, sink); }, 500);
+  double seen0, cnt0, seen32, cnt32;
+  run_fetch_behind_stores<0>(&seen0, &cnt0);
+  run_fetch_behind_stores<32>(&seen32, &cnt32);
+  printf("{\"fetch_behind_stores\": {\"unit\": \"shader-clock cycles, mean over 256 waves\", "
+         "\"alone\": {\"data_visible_in_lds\": %.0f, \"vmcnt_0\": %.0f}, "
+         "\"behind_32_stores\": {\"data_visible_in_lds\": %.0f, \"vmcnt_0\": %.0f}}}\n", seen0, cnt0, seen32, cnt32);
   printf("{\"launch_cost\": {\"period_us\": {\"empty_1_block\": %.2f, \"empty_256_blocks\": %.2f, \"empty_256_blocks_64KiB_lds\": %.2f, "
          "\"write_64MiB\": %.2f, \"write_64MiB_as_gemm_tiles_64B_per_row\": %.2f, \"write_64MiB_as_gemm_tiles_128B_per_row\": %.2f, "
          "\"same_64B_nontemporal\": %.2f, \"same_128B_nontemporal\": %.2f}, \"write_GBps\": %.0f, "

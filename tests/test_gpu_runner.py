@@ -128,7 +128,13 @@ def test_runner_launch_cost_mode():
     64 MiB (the fp32 result of a 4096 x 4096 product) takes at least what 8 TB/s of HBM allow."""
     p = _run(["--launch-cost"])
     assert p.returncode == 0
-    r = json.loads(p.stdout.strip().splitlines()[-1])["launch_cost"]
+    lines = p.stdout.strip().splitlines()
+    f = json.loads(lines[-2])["fetch_behind_stores"]
+    # a fetch lands, and is reported, no earlier behind 32 stores of the same wave than alone; the counter never
+    # reports before the data is there
+    assert 0 < f["alone"]["data_visible_in_lds"] <= f["alone"]["vmcnt_0"]
+    assert f["alone"]["data_visible_in_lds"] <= f["behind_32_stores"]["data_visible_in_lds"] <= f["behind_32_stores"]["vmcnt_0"]
+    r = json.loads(lines[-1])["launch_cost"]
     per = r["period_us"]
     assert 0.5 < per["empty_1_block"] < 50.0 and 0.5 < per["empty_256_blocks"] < 50.0
     assert per["write_64MiB"] > (64 << 20) / 8e12 * 1e6
