@@ -26,7 +26,7 @@
 
 #include "kcg_config.h"
 
-#define KCG_VERSION "kcg-gemm-gfx950 0.1"
+#define KCG_VERSION "kcg-gemm-gfx950 0.2"
 
 // The device template headers, embedded at build time (directory given by -DKCG_DEVICE_HEADER_DIR):
 // kcg_gemm_device.h is what the instantiation stub includes; it includes the others.
@@ -459,6 +459,7 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
     flags_text += "hiprtc" + std::to_string(major) + "." + std::to_string(minor);
   }
   for (const auto& f : extra_flags()) flags_text += f + " ";
+  if (!env_flag("KCG_SPILL_REBUILD", true)) flags_text += "first-build-kept ";
   uint64_t h = fnv1a(KCG_VERSION);
   h = fnv1a(arch, h);
   h = fnv1a(flags_text, h);
@@ -484,31 +485,38 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
     if (direct && file_exists(spill_marker)) return kBuildSpills;
   }
 
-  hiprtcProgram prog;
-  hiprtcResult r = RTCF(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", kNumDeviceHeaders,
-                                             const_cast<const char**>(kDeviceHeaderSrcs),
-                                             const_cast<const char**>(kDeviceHeaderNames));
-  if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTCF(hiprtcGetErrorString)(r));
-  std::vector<std::string> opts = compile_flags();
-  opts.push_back("--offload-arch=" + arch);
-  for (const auto& f : extra_flags()) opts.push_back(f);
-  std::vector<const char*> optv;
-  for (const auto& o : opts) optv.push_back(o.c_str());
-  r = RTCF(hiprtcCompileProgram)(prog, (int)optv.size(), optv.data());
-  if (r != HIPRTC_SUCCESS) {
+  // one hiprtc build of the stub with the engine's flags, $KCG_EXTRA_FLAGS and `more` behind them
+  auto compile = [&](const std::vector<std::string>& more, std::vector<char>* code) -> int {
+    hiprtcProgram prog;
+    hiprtcResult r = RTCF(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", kNumDeviceHeaders,
+                                               const_cast<const char**>(kDeviceHeaderSrcs),
+                                               const_cast<const char**>(kDeviceHeaderNames));
+    if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTCF(hiprtcGetErrorString)(r));
+    std::vector<std::string> opts = compile_flags();
+    opts.push_back("--offload-arch=" + arch);
+    for (const auto& f : extra_flags()) opts.push_back(f);
+    for (const auto& f : more) opts.push_back(f);
+    std::vector<const char*> optv;
+    for (const auto& o : opts) optv.push_back(o.c_str());
+    r = RTCF(hiprtcCompileProgram)(prog, (int)optv.size(), optv.data());
+    if (r != HIPRTC_SUCCESS) {
+      size_t n = 0;
+      RTCF(hiprtcGetProgramLogSize)(prog, &n);
+      std::string log(n, 0);
+      if (n) RTCF(hiprtcGetProgramLog)(prog, &log[0]);
+      RTCF(hiprtcDestroyProgram)(&prog);
+      return fail(KCG_ERR_COMPILE, std::string("hiprtc: ") + RTCF(hiprtcGetErrorString)(r) + " for " + name + "\n" + log);
+    }
     size_t n = 0;
-    RTCF(hiprtcGetProgramLogSize)(prog, &n);
-    std::string log(n, 0);
-    if (n) RTCF(hiprtcGetProgramLog)(prog, &log[0]);
+    r = RTCF(hiprtcGetCodeSize)(prog, &n);
+    code->assign(n, 0);
+    if (r == HIPRTC_SUCCESS) r = RTCF(hiprtcGetCode)(prog, code->data());
     RTCF(hiprtcDestroyProgram)(&prog);
-    return fail(KCG_ERR_COMPILE, std::string("hiprtc: ") + RTCF(hiprtcGetErrorString)(r) + " for " + name + "\n" + log);
-  }
-  size_t n = 0;
-  r = RTCF(hiprtcGetCodeSize)(prog, &n);
-  std::vector<char> code(n);
-  if (r == HIPRTC_SUCCESS) r = RTCF(hiprtcGetCode)(prog, code.data());
-  RTCF(hiprtcDestroyProgram)(&prog);
-  if (r != HIPRTC_SUCCESS || n == 0) return fail(KCG_ERR_COMPILE, "hiprtc returned no code object");
+    if (r != HIPRTC_SUCCESS || n == 0) return fail(KCG_ERR_COMPILE, "hiprtc returned no code object");
+    return KCG_OK;
+  };
+  std::vector<char> code;
+  if (int rc = compile({}, &code)) return rc;
   // The direct-staging kernel reads LDS with instructions the compiler does not know to be
   // asynchronous: a fragment register spilled to scratch memory would be stored before its data has
   // arrived.  Such a build is never used (nor cached): the caller falls back to register staging.
@@ -517,6 +525,17 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
     const char note[] = "direct-staging build needs scratch memory (register spills); register staging is used instead\n";
     write_file_atomic(spill_marker, note, sizeof(note) - 1);
     return kBuildSpills;
+  }
+  // A register-staged or scalar kernel that does not fit the register file without spilling is built once
+  // more at -O1, and that build is the one kept.  One such kernel (fp64, one wave on a 64x64x64 tile with
+  // both prefetch flags, M=8 N=208 K=592: 512 registers and 1 KiB of scratch per lane) returns wrong sums at
+  // -O2 and -O3 and the right ones at -O1, as do all spilling kernels of a 1000-config random sample (184 of
+  // them, 9 % slower at the median).  Such configs never win a tuning run; they must still be right.
+  // $KCG_SPILL_REBUILD=0 keeps the first build.
+  if (!direct && code_object_scratch_bytes(code) != 0 && env_flag("KCG_SPILL_REBUILD", true)) {
+    std::vector<char> calm;
+    if (int rc = compile({"-O1"}, &calm)) return rc;
+    code.swap(calm);
   }
   if (!write_file_atomic(path, code.data(), code.size())) return fail(KCG_ERR_IO, "cannot write " + path);
   if (env_flag("KCG_KEEP_SOURCE", false)) {

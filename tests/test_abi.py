@@ -109,3 +109,27 @@ def test_direct_staging_build_that_spills_falls_back_to_register_staging(tmp_pat
     assert "static constexpr bool DIRECT = false;" not in _native.instantiation_source(values, _native.KIND_MFMA)
     again = _native.compile_matmul(values, "gfx950", _native.KIND_MFMA)                 # marker + cache: nothing is compiled
     assert again["cache_hit"] and again["code_path"] == info["code_path"]
+
+
+def test_register_staged_build_that_spills_is_rebuilt_at_a_lower_optimisation_level(tmp_path, monkeypatch):
+    """A scalar or register-staged kernel that needs scratch memory is built a second time at -O1 and that
+    build is the one kept ($KCG_SPILL_REBUILD=0 keeps the first; the switch is part of the cache key).  A
+    kernel without spills is built once, whatever the switch says."""
+    monkeypatch.setenv("KCG_CACHE_DIR", str(tmp_path))
+    # fp32 scalar kernel, one wave on a 32x32x64 tile, edge tiles everywhere: spills at -O3 (a case of the random samples)
+    spilling = [32, 32, 64, 4, 4, 64, 1, 1, 8, 8, 4, 4, 4, 4, 4, 4, 1, 2, 4, 4, 1, 1, 1, 1, 4, 4, 4, 435, 401, 487, 1]
+    calm = [64, 64, 16, 4, 4, 64, 2, 2, 8, 8, 4, 4, 4, 4, 4, 4, 1, 8, 4, 4, 0, 0, 0, 1, 4, 4, 4, 1024, 1024, 1024, 1]
+
+    def build(values):
+        info = _native.compile_matmul(values, "gfx950", _native.KIND_SIMT)
+        with open(info["code_path"], "rb") as f:
+            return info["code_path"], f.read()
+
+    p_spill, code_spill = build(spilling)
+    p_calm, code_calm = build(calm)
+    monkeypatch.setenv("KCG_SPILL_REBUILD", "0")
+    p_spill_first, code_spill_first = build(spilling)
+    p_calm_first, code_calm_first = build(calm)
+    assert p_spill != p_spill_first and p_calm != p_calm_first          # the switch is part of the cache key
+    assert code_spill != code_spill_first                               # the kept build is another one
+    assert code_calm == code_calm_first                                 # nothing to rebuild

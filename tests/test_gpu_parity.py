@@ -286,8 +286,15 @@ def extra_build_configs():
     bf16 = dict(_tuned("gemm_4096_fp16.json"))
     bf16["DATATYPE_A"] = bf16["DATATYPE_B"] = 3
     out.append((bf16, 0))
+    out.append((SPILLING_FP64_CONFIG, MFMA))
     return out
 
+
+# fp64, one wave on a 64x64x64 tile with both prefetch flags, edge tiles in M and N and a partial last K tile:
+# the register-staged kernel cannot fit the register file (512 registers and scratch memory besides), and its
+# build at the usual optimisation level returned wrong sums in the last block column
+SPILLING_FP64_CONFIG = dict(zip(_native.keywords(), [64, 64, 64, 4, 16, 64, 1, 1, 16, 4, 2, 2, 2, 2, 2, 2, 1, 4, 2, 4, 1, 1,
+                                                      0, 1, 8, 8, 8, 8, 208, 592, 0]))
 
 CONFIG4_KERNELS = ((MFMA, dict(BM=128, BN=128, TM=8, TN=8, BK=16, shared_prefetch=1, is_atrans=0)),
                    (MFMA, dict(BM=64, BN=64, BK=32, is_atrans=1)),
@@ -455,3 +462,14 @@ def test_tuned_edge_shape_kernels_are_bit_exact_on_integers(oracle, index):
     assert not np.isnan(got).any()
     bad = np.argwhere(got != want)
     assert bad.size == 0, f"tuned edge config {index}: {len(bad)} mismatches, first at {bad[:5].tolist()}"
+
+
+def test_kernel_that_needs_scratch_memory_is_exact(oracle):
+    """A register-staged kernel whose first build spills registers is built again at a lower optimisation
+    level by the engine; the kernel it hands out is bit-exact on integers (and still reports its scratch use)."""
+    from tests.gemm_helpers import build_kernel
+    kpm, ui, kernel, info = build_kernel(SPILLING_FP64_CONFIG, MFMA)
+    assert info["kind"] == MFMA and info["lds_bytes"] > 0          # register staging: fp64 has no direct-staging form
+    assert kernel.n_spills > 0
+    kernel.unload()
+    _exact_case(oracle, SPILLING_FP64_CONFIG, MFMA, "mfma-f64-one-wave-64x64x64-spilling")
