@@ -21,7 +21,9 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "kcg_config.h"
@@ -52,6 +54,23 @@ static const int kNumDeviceHeaders = 6;
 namespace {
 
 thread_local std::string g_err;
+
+// Functions handed out by kcg_load: which argument list their kernel takes (3: the reference's three pointers,
+// 8: the batched-strided form) and which module owns them.  kcg_launch / kcg_launch_batched refuse a known
+// function of the other form instead of starting a kernel on a parameter block it would misread; a handle
+// that did not come from kcg_load is launched as the caller says.
+struct LoadedFunction {
+  int n_args;
+  uint64_t module;
+};
+std::mutex g_loaded_mu;
+std::unordered_map<uint64_t, LoadedFunction> g_loaded;
+
+int loaded_args(uint64_t function) {
+  std::lock_guard<std::mutex> lock(g_loaded_mu);
+  auto it = g_loaded.find(function);
+  return it == g_loaded.end() ? 0 : it->second.n_args;
+}
 
 int fail(int code, const std::string& msg) {
   g_err = msg;
@@ -603,6 +622,15 @@ int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int 
   if (n_spills) *n_spills = local / 4;   // scratch dwords per lane; 0 means no spilling
   *module = (uint64_t)(uintptr_t)mod;
   *function = (uint64_t)(uintptr_t)fn;
+  {
+    const std::string name(kernel_name);
+    auto ends = [&](const char* suffix) {
+      const size_t n = strlen(suffix);
+      return name.size() >= n && name.compare(name.size() - n, n, suffix) == 0;
+    };
+    std::lock_guard<std::mutex> lock(g_loaded_mu);
+    g_loaded[*function] = LoadedFunction{(ends("EX_") || ends("EXab_")) ? 8 : 3, *module};
+  }
   g_err.clear();
   return KCG_OK;
 }
@@ -612,6 +640,7 @@ int kcg_launch(uint64_t function, const int32_t grid[3], const int32_t block[3],
   if (!function || !grid || !block) return fail(KCG_ERR_ARGUMENT, "null function / dims");
   if ((int64_t)grid[0] * grid[1] * grid[2] <= 0) return KCG_OK;  // empty grid: nothing to do
   if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
+  if (loaded_args(function) == 8) return fail(KCG_ERR_ARGUMENT, "this kernel has the batched-strided form: use kcg_launch_batched");
   void* pa = (void*)(uintptr_t)a;
   void* pb = (void*)(uintptr_t)b;
   void* pc = (void*)(uintptr_t)c;
@@ -632,6 +661,7 @@ int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t b
   if ((int64_t)grid[0] * grid[1] * grid[2] <= 0 || batch == 0) return KCG_OK;  // nothing to do
   if (grid[1] != 1 || grid[2] != 1) return fail(KCG_ERR_ARGUMENT, "the batch goes on grid[1]: grid must be {n, 1, 1}");
   if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
+  if (loaded_args(function) == 3) return fail(KCG_ERR_ARGUMENT, "this kernel has the three-pointer form: use kcg_launch");
   void* pa = (void*)(uintptr_t)a;
   void* pb = (void*)(uintptr_t)b;
   void* pc = (void*)(uintptr_t)c;
@@ -706,6 +736,10 @@ int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[
 int kcg_unload(uint64_t module) {
   if (!module) return fail(KCG_ERR_ARGUMENT, "null module");
   HIP_READY();
+  {
+    std::lock_guard<std::mutex> lock(g_loaded_mu);
+    for (auto it = g_loaded.begin(); it != g_loaded.end();) it = it->second.module == module ? g_loaded.erase(it) : std::next(it);
+  }
   HIP_TRY(HIPF(hipModuleUnload)((hipModule_t)(uintptr_t)module));
   return KCG_OK;
 }

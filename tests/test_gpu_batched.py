@@ -164,7 +164,18 @@ def test_launch_batched_argument_checks():
         kernel.run(a, b, c)                                                # the three-pointer launch does not fit this kernel
     kernel.run_batched(a, b, c, 0, 0, 0, 0)                                # empty batch: nothing launched
     torch.cuda.synchronize()
+    # the C ABI itself knows which form a function it loaded has, and refuses the other launch call
+    ui = kernel.m_launcher.m_kernelLib
+    fn = kernel.m_launcher._function()
+    with pytest.raises(_native.KcgError, match="kcg_launch_batched"):
+        _native.launch(fn, ui.m_gridDims, ui.m_blockDims, ui.m_shmSize, 0, a.data_ptr(), b.data_ptr(), c.data_ptr())
     kernel.unload()
     _, plain, _ = build(cfg, SIMT, None)
     with pytest.raises(TypeError):
         plain.run_batched(a, b, c, 1, 0, 0, 0)
+    ui = plain.m_launcher.m_kernelLib
+    fn = plain.m_launcher._function()
+    with pytest.raises(_native.KcgError, match="kcg_launch"):
+        _native.launch_batched(fn, ui.m_gridDims, ui.m_blockDims, ui.m_shmSize, 0, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+                               1, 0, 0, 0)
+    plain.unload()
