@@ -219,7 +219,7 @@ int reference_lds_bytes(const MatmulConfig& c) {
 // Must state the same rule as DirectPlan<C>::ELIGIBLE in kcg_device_direct.h (a static_assert there
 // compares the two): 16-bit inputs or fp32 throughout, at least one full K tile, both prefetch flags, LOAD_CONTINUOUS, 128-bit load
 // widths, tiles (powers of two or multiples of 16 chunks) that split evenly into 1 KiB wave fetches, at least two rows of
-// matrix-core tiles per wave, two LDS stages within 160 KiB, and M, N, K multiples of the 16-byte vector unless the elements have 4 bytes.
+// matrix-core tiles per wave, two LDS stages within 160 KiB; any M, N and K >= BK.
 bool mfma_direct(const MatmulConfig& c) {
   MfmaPlan p = plan_mfma(c);
   const int es = dtype_size(c.dtA);
@@ -240,10 +240,8 @@ bool mfma_direct(const MatmulConfig& c) {
   auto tile_ok = [g](int x) { return is_pow2(x) || (x > 0 && x % (16 * g) == 0); };
   if (!tile_ok(c.BM) || !tile_ok(c.BN) || !is_pow2(c.BK) || c.BM < 32 || c.BN < 32) return false;
   if ((c.BM * c.BK / g) % (64 * nw) || (c.BN * c.BK / g) % (64 * nw)) return false;
-  // rows of A and B that do not start on 16-byte boundaries: fetched in 4-byte pieces (one fp32 element, two 16-bit
-  // elements), which must not straddle a row end
-  const int piece = 4 / es;                               // (es is 2 or 4 here)
-  if ((c.M % g || c.N % g || c.K % g) && (c.M % piece || c.N % piece || c.K % piece)) return false;
+  // (rows of A and B that do not start on 16-byte boundaries are fetched in 4-byte pieces: one fp32 element, or two
+  // 16-bit elements from an even column on, whatever the extents)
   const long lim = 1L << 31;                              // 32-bit byte offsets per lane inside a tile panel
   if ((long)c.BM * c.K * es >= lim || (long)c.BK * c.M * es >= lim || (long)c.BK * c.N * es >= lim) return false;
   return 2 * (c.BM + c.BN) * c.BK * es <= kMaxLdsBytes;

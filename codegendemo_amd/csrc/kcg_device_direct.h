@@ -152,11 +152,21 @@ struct DirectPlan {
   static constexpr bool tile_ok(int x) { return pow2(x) || (x > 0 && x % (16 * G) == 0); }
   // What a lane fetches: a whole 16-byte chunk where every row of A and B starts on a 16-byte boundary (M, N and K
   // multiples of G); otherwise 4 bytes (the same instruction with a 4-byte payload: a wave's 64 pieces land in 256
-  // consecutive bytes of LDS) — one 4-byte element, or two 2-byte elements where M, N and K are even.
+  // consecutive bytes of LDS) — one 4-byte element, or the two 2-byte elements at an even and the next odd column.
+  // With 16-bit rows of odd length every other row starts 2 bytes off a 4-byte boundary; the fetch takes such
+  // source addresses (at about 60 % of the aligned rate), and the piece at the end of a row brings the first
+  // element of the next row with it, which lands in a column (or k value) that does not exist and is never used.
   static constexpr bool CHUNK_FETCH = C::M % G == 0 && C::N % G == 0 && C::K % G == 0;
   static constexpr int FGMIN = ES <= 4 ? 4 / ES : 1;              // elements in 4 bytes
-  static constexpr bool PIECE_FETCH = ES <= 4 && C::M % FGMIN == 0 && C::N % FGMIN == 0 && C::K % FGMIN == 0;
+  static constexpr bool PIECE_FETCH = ES <= 4;
   static constexpr int FG = CHUNK_FETCH ? G : FGMIN;              // elements per lane and fetch instruction
+  // The piece that holds the last element of a matrix with odd rows would reach 2 bytes past the end of the buffer
+  // when it starts 2 bytes off a 4-byte boundary, i.e. when the matrix has an even number of rows; past the end may
+  // be another page.  Such a matrix gets its last piece from 2 bytes further down, and the lane that fetched it
+  // moves the element into place in LDS (see patch_final in the kernel).
+  static constexpr int A_ROWS = C::ATRANS ? C::K : C::M, A_COLS = C::ATRANS ? C::M : C::K;
+  static constexpr bool FIX_A = ES == 2 && A_COLS % 2 == 1 && A_ROWS % 2 == 0;
+  static constexpr bool FIX_B = ES == 2 && C::N % 2 == 1 && C::K % 2 == 0;
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
@@ -213,6 +223,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int KT = K / BK;                            // full K tiles
   constexpr int KR = K % BK, SPWT = cdiv(KR, KS);       // the remainder: one more tile of SPWT k-steps (the last may be partial)
   constexpr int KTT = KT + (KR > 0 ? 1 : 0);
+  // The last tile computes its fetch offsets on the spot instead of taking the registers all other tiles share,
+  // when it is the partial one or holds a piece that is fetched from another place (FIX_A / FIX_B).
+  // KTF: tiles in front of it; KLAST: its k extent.
+  constexpr bool FINAL_SPECIAL = KR > 0 || P::FIX_A || P::FIX_B;
+  constexpr int KTF = FINAL_SPECIAL ? KTT - 1 : KTT;
+  constexpr int KLAST = KR > 0 ? KR : BK;
   constexpr bool EDGE_M = M % BM != 0, EDGE_N = N % BN != 0;
   constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
   constexpr int ES = P::ES, G = P::G;                   // element size; elements per 16-byte chunk
@@ -267,37 +283,48 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
   // never changes: the K loop spends no vector instruction on addresses.
   // kvalid: how many k rows/values of the tile exist (BK, or KR for the partial tile)
-  auto off_a = [&](int idx, int kvalid) -> unsigned {
+  // fix: the tile is the last one of the K loop and the piece with the matrix's last element is taken from 2 bytes
+  // further down (DirectPlan::FIX_A / FIX_B); *moved (optional) says whether this lane's piece is that one
+  auto off_a = [&](int idx, int kvalid, bool fix = false, bool* moved = nullptr) -> unsigned {
     const int p = 64 * (wave * NIA + idx) + lane;     // physical fetch-granule slot inside the A stage
     const int s = p / GPC, e = (p % GPC) * FG;        // chunk slot; first element of the granule inside its chunk
+    bool last = false;
+    unsigned off;
     if constexpr (AK) {
       int row = s / CHK;
       const int cp = s % CHK;
       const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
       int k = c * G + e;
-      if (k >= kvalid) k = 0;
       if constexpr (EDGE_M) row = cmin(row, M - 1 - m0);
-      return (unsigned)((row * K + k) * ES);
+      last = P::FIX_A && fix && m0 + row == M - 1 && k == kvalid - 1;
+      if (k >= kvalid) k = 0;
+      off = (unsigned)((row * K + k) * ES);
     } else {
       int k = s / NCHA;
       const int cp = s % NCHA;
       const int c = cp ^ swz_n(k, NCHA);
       int m = c * G + e;
+      if constexpr (EDGE_M) m = cmin(m, ((M - m0 - 1) / FG) * FG);   // the last piece that starts inside the row
+      last = P::FIX_A && fix && k == kvalid - 1 && m0 + m == M - 1;
       if (k >= kvalid) k = 0;
-      if constexpr (EDGE_M) m = cmin(m, M - m0 - FG);
-      return (unsigned)((k * M + m) * ES);
+      off = (unsigned)((k * M + m) * ES);
     }
+    if (moved) *moved = last;
+    return last ? off - ES : off;
   };
-  auto off_b = [&](int j, int kvalid) -> unsigned {
+  auto off_b = [&](int j, int kvalid, bool fix = false, bool* moved = nullptr) -> unsigned {
     const int p = 64 * (wave * NIB + j) + lane;
     const int s = p / GPC, e = (p % GPC) * FG;
     int k = s / NCHB;
     const int cp = s % NCHB;
     const int c = cp ^ swz_n(k, NCHB);
     int n = c * G + e;
+    if constexpr (EDGE_N) n = cmin(n, ((N - n0 - 1) / FG) * FG);
+    const bool last = P::FIX_B && fix && k == kvalid - 1 && n0 + n == N - 1;
     if (k >= kvalid) k = 0;
-    if constexpr (EDGE_N) n = cmin(n, N - n0 - FG);
-    return (unsigned)((k * N + n) * ES);
+    if (moved) *moved = last;
+    const unsigned off = (unsigned)((k * N + n) * ES);
+    return last ? off - ES : off;
   };
   unsigned voff_a[NIA], voff_b[NIB];
 #pragma unroll
@@ -318,13 +345,13 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     asm("" : "+s"(t.a), "+s"(t.b));
     return t;
   };
-  // partial_c: the tile fetched is the partial one behind the last full K tile
+  // partial_c: the tile fetched is the last one and FINAL_SPECIAL
   auto fetch_item = [&](int idx, const TileBase& tb, auto stage_c, auto partial_c) {
     constexpr bool PARTIAL = decltype(partial_c)::value;
     char* st = stage_ptr(stage_c);
     if (idx < NIA) {
       unsigned off;
-      if constexpr (PARTIAL) off = off_a(idx, KR);
+      if constexpr (PARTIAL) off = off_a(idx, KLAST, true);
       else {
         asm volatile("" : "+v"(voff_a[idx]));   // keeps the 32->64 bit extension next to the fetch (see tile_base)
         off = voff_a[idx];
@@ -335,7 +362,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     } else {
       const int j = idx - NIA;
       unsigned off;
-      if constexpr (PARTIAL) off = off_b(j, KR);
+      if constexpr (PARTIAL) off = off_b(j, KLAST, true);
       else {
         asm volatile("" : "+v"(voff_b[j]));
         off = voff_b[j];
@@ -346,6 +373,40 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     }
   };
   constexpr int NFETCH = NIA + NIB;
+  // FIX_A / FIX_B: the piece with the last element of the matrix was fetched from 2 bytes further down, so its
+  // 32-bit word in LDS holds the last element in the upper half.  The lane that fetched it shifts it down (what
+  // the upper half then stands for does not exist: a column beyond N, a row beyond M or a k value beyond K).
+  // Called by every wave once its own fetches of the last tile have landed, in front of the barrier that
+  // publishes the tile.
+  auto patch_final = [&](auto stage_c) {
+    const unsigned st = (unsigned)(unsigned long)stage_ptr(stage_c);
+    auto shift_down = [&](unsigned addr) {
+      unsigned w;
+      asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(w) : "v"(addr) : "memory");
+      w >>= 16;
+      asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(addr), "v"(w) : "memory");
+    };
+    if constexpr (P::FIX_A) {
+      if (m0 + BM >= M) {                       // (the block row with the last row of A, or its last column)
+#pragma unroll
+        for (int idx = 0; idx < NIA; ++idx) {
+          bool moved;
+          (void)off_a(idx, KLAST, true, &moved);
+          if (moved) shift_down(st + (unsigned)(FETCH_BYTES * (wave * NIA + idx) + lane * 4));
+        }
+      }
+    }
+    if constexpr (P::FIX_B) {
+      if (n0 + BN >= N) {
+#pragma unroll
+        for (int j = 0; j < NIB; ++j) {
+          bool moved;
+          (void)off_b(j, KLAST, true, &moved);
+          if (moved) shift_down(st + (unsigned)(A_BYTES + FETCH_BYTES * (wave * NIB + j) + lane * 4));
+        }
+      }
+    }
+  };
 
   // ---- fragments -----------------------------------------------------------------------------
   // Every fragment read is issued as inline assembly.  As builtins or plain loads the compiler could
@@ -358,14 +419,21 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   const int frow = lane % MF, fgrp = lane / MF;
   const int tx = lane % 16;                          // lane inside its 16-lane transposing group
   const int tsub = (lane / 16) % (MF / 16);          // which 16-column half of the matrix-core tile
+  // a 32-bit word of two 16-bit k values of which the first `left` exist (K even: left is even, the middle case never occurs)
+  struct Pair16 {
+    __device__ __forceinline__ static unsigned keep(unsigned w, int left) {
+      if constexpr (K % 2 == 0) return left > 0 ? w : 0u;
+      else return left > 1 ? w : (left == 1 ? (w & 0xFFFFu) : 0u);
+    }
+  };
   struct FragTr {                                    // 16-bit, row-contiguous tile: two transposing 64-bit reads
     u32x2 h[2];
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(h[0]), "+v"(h[1])); }
-    // nvalid: how many of the lane's G = 8 consecutive k values exist (an even number: K is even).  h[0] holds
-    // k values 0..3 of them (two per 32-bit word), h[1] the values 4..7.
+    // nvalid: how many of the lane's G = 8 consecutive k values exist.  h[0] holds k values 0..3 of them (two per
+    // 32-bit word, the earlier one in the lower half), h[1] the values 4..7.
     __device__ __forceinline__ void keep_first(int nvalid) {
-      h[0].x = 0 < nvalid ? h[0].x : 0u; h[0].y = 2 < nvalid ? h[0].y : 0u;
-      h[1].x = 4 < nvalid ? h[1].x : 0u; h[1].y = 6 < nvalid ? h[1].y : 0u;
+      h[0].x = Pair16::keep(h[0].x, nvalid - 0); h[0].y = Pair16::keep(h[0].y, nvalid - 2);
+      h[1].x = Pair16::keep(h[1].x, nvalid - 4); h[1].y = Pair16::keep(h[1].y, nvalid - 6);
     }
     __device__ __forceinline__ Frag get() const {
       const u32x4 v = {h[0].x, h[0].y, h[1].x, h[1].y};
@@ -390,8 +458,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     __device__ __forceinline__ void keep_first(int nvalid) {
       if constexpr (ES == 4) {                                      // one k value per 32-bit word
         q.x = 0 < nvalid ? q.x : 0u; q.y = 1 < nvalid ? q.y : 0u; q.z = 2 < nvalid ? q.z : 0u; q.w = 3 < nvalid ? q.w : 0u;
-      } else {                                                      // two k values per 32-bit word, K is even
-        q.x = 0 < nvalid ? q.x : 0u; q.y = 2 < nvalid ? q.y : 0u; q.z = 4 < nvalid ? q.z : 0u; q.w = 6 < nvalid ? q.w : 0u;
+      } else {                                                      // two k values per 32-bit word
+        q.x = Pair16::keep(q.x, nvalid - 0); q.y = Pair16::keep(q.y, nvalid - 2); q.z = Pair16::keep(q.z, nvalid - 4); q.w = Pair16::keep(q.w, nvalid - 6);
       }
     }
     __device__ __forceinline__ Frag get() const { return __builtin_bit_cast(Frag, q); }
@@ -478,7 +546,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   static_for<0, NST>([&](auto t) {
     if (decltype(t)::value < KTT) {
 #pragma unroll
-      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t, BoolC<(KR > 0 && decltype(t)::value == KT)>());
+      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t, BoolC<(FINAL_SPECIAL && decltype(t)::value == KTF)>());
     }
   });
 
@@ -535,6 +603,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int NPRO = cmin(NST, KTT);                                    // tiles the prologue has issued
   __builtin_amdgcn_s_waitcnt(vmcnt_only(cmin(63, (NPRO - 1) * NFETCH)));  // this wave's chunks of tile 0 are in LDS
   asm volatile("" ::: "memory");
+  if constexpr ((P::FIX_A || P::FIX_B) && KTT == 1) patch_final(IntC<0>());
   __builtin_amdgcn_s_barrier();                                            // ... and everyone's (bare barrier: see the K loop)
   asm volatile("" ::: "memory");
 #if KCG_TIMELINE
@@ -559,7 +628,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // takes 16 cycles per 1 KiB fetch instruction; four waves issuing all of theirs right behind the
   // barrier would stall on it); with two stages they must all be issued in the rest of this tile.
   constexpr int SPREAD = NST >= 3 ? MT : TAIL;
-  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c, auto ns_c, auto pn_c, auto pp_c) {
+  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c, auto ns_c, auto pn_c, auto pp_c, auto fixn_c) {
     constexpr int CUR = decltype(cur_c)::value, NS = decltype(ns_c)::value;
     constexpr int NXT = (CUR + 1) % NST, PRV = (CUR + NST - 1) % NST;
     constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
@@ -592,6 +661,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 #endif
           if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
           wait_lds();        // this wave's reads of stage CUR have all returned
+          if constexpr (decltype(fixn_c)::value) patch_final(IntC<NXT>());   // tile kt+1 is the last one (nothing behind it in flight)
           // ... everyone's part; and every wave is done reading stage CUR.  The bare barrier instruction:
           // __syncthreads() comes with a fence in front of which the compiler drains every fetch in
           // flight (vmcnt(0)), which would expose the whole memory latency at each tile.  What has
@@ -664,20 +734,22 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // tiles_ahead(T): how many tiles behind tile T+1 have been issued when tile T reaches its barrier
   // (the prologue issued tiles 0..NST-1, tile t issues or completes the issue of tile t-1+NST)
   typedef BoolC<false> No;
-  tile(0, IntC<0>(), BoolC<(1 < KTT)>(), BoolC<(NST < KTT)>(), No(), IntC<tiles_ahead(0)>(), IntC<SPW>(),
-       BoolC<(KR > 0 && NST == KT)>(), No());
-  constexpr int NFULL = KT - NST - 1 > 0 ? KT - NST - 1 : 0;   // tiles 1 .. KT-NST-1 have kt+NST < KT: full tiles all round
+  constexpr bool FIX = P::FIX_A || P::FIX_B;
+  tile(0, IntC<0>(), BoolC<(1 < KTT)>(), BoolC<(NST < KTT)>(), No(), IntC<tiles_ahead(0)>(), IntC<(0 < KT ? SPW : SPWT)>(),
+       BoolC<(FINAL_SPECIAL && NST == KTF)>(), No(), BoolC<(FIX && 2 == KTT)>());
+  constexpr int NFULL = KTF - NST - 1 > 0 ? KTF - NST - 1 : 0;   // tiles 1 .. KTF-NST-1 have kt+NST < KTF: ordinary tiles all round
   constexpr int NG = NFULL / NST;
   for (int g = 0; g < NG; ++g) {
     static_for<0, NST>([&](auto sc) {
       constexpr int S = decltype(sc)::value;
-      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>(), IntC<SPW>(), No(), No());
+      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>(), IntC<SPW>(), No(), No(), No());
     });
   }
   static_for<1 + NG * NST, KTT>([&](auto tc) {
     constexpr int T = decltype(tc)::value;
     tile(T, IntC<T % NST>(), BoolC<(T + 1 < KTT)>(), BoolC<(T + NST < KTT)>(), BoolC<(T - 1 + NST < KTT)>(), IntC<tiles_ahead(T)>(),
-         IntC<(T < KT ? SPW : SPWT)>(), BoolC<(KR > 0 && T + NST == KT)>(), BoolC<(KR > 0 && T - 1 + NST == KT)>());
+         IntC<(T < KT ? SPW : SPWT)>(), BoolC<(FINAL_SPECIAL && T + NST == KTF)>(), BoolC<(FINAL_SPECIAL && T - 1 + NST == KTF)>(),
+         BoolC<(FIX && T + 2 == KTT)>());
   });
 
   // the last matrix-core results must have left the pipeline before the epilogue reads them (the

@@ -192,6 +192,82 @@ def random_even_16bit_direct_configs(n=20, seed=20251126):
     return out
 
 
+def odd16_class(cfg):
+    """Which special case of 16-bit rows of odd length a config exercises: 'a-kcont' / 'a-rowcont' / 'b' — the last
+    piece of that operand would reach past the buffer and is fetched from 2 bytes further down; 'k-odd' — the last
+    k value shares its 32-bit word with one that does not exist; 'plain' — odd rows, none of these."""
+    M, N, K, at = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"], cfg["IS_ATRANS"]
+    out = []
+    if not at and K % 2 == 1 and M % 2 == 0:
+        out.append("a-kcont")
+    if at and M % 2 == 1 and K % 2 == 0:
+        out.append("a-rowcont")
+    if N % 2 == 1 and K % 2 == 0:
+        out.append("b")
+    if K % 2 == 1:
+        out.append("k-odd")
+    return out or ["plain"]
+
+
+def random_odd_16bit_direct_configs(n=36, seed=20251127):
+    """-> [(config, kind)]: fp16 / bf16 configs with an odd M, N or K that take the direct-staging kernel (rows that
+    start 2 bytes off a 4-byte boundary), at least six of each class of odd16_class, K remainders of any length
+    (also none: the last row of B then sits in a full tile), both A layouts, 16-bit and fp32 outputs."""
+    rng = random.Random(seed)
+    out, seen = [], {}
+    while len(out) < n or min(seen.get(c, 0) for c in ("a-kcont", "a-rowcont", "b", "k-odd")) < 6:
+        dtype = rng.choice([2, 3])
+        BM, BN = rng.choice([32, 64, 128, 256]), rng.choice([32, 64, 128, 256])
+        BK = rng.choice([16, 32, 64])
+        out16 = rng.random() < 0.3
+        kt = rng.choice([1, 2, 3] if out16 else [1, 2, 3, 4, 5, 7, 9, 12])
+        kw = dict(BM=BM, BN=BN, BK=BK, TM=rng.choice([2, 4, 8, 16]), TN=rng.choice([2, 4, 8, 16]),
+                  warp_layout=rng.choice([(8, 8), (8, 8), (4, 16), (16, 4)]), dtype=dtype, dtype_c=dtype if out16 else 4,
+                  is_atrans=rng.choice([0, 1]), block_mapping=rng.choice([0, 2, 4, 8]), shared_prefetch=1, reg_prefetch=1,
+                  M=BM * rng.choice([1, 2]) - rng.choice([0, 1, 2, 3, 5, 8, BM - 1, BM // 2 + 1]),
+                  N=BN * rng.choice([1, 2, 3]) - rng.choice([0, 1, 2, 3, 7, 8, BN - 1, BN // 2 - 1]),
+                  K=BK * kt + rng.choice([0, 0, 1, 2, 3, 5, 8, 13, 31]) % BK)
+        if kw["M"] <= 0 or kw["N"] <= 0 or (kw["M"] % 2 == 0 and kw["N"] % 2 == 0 and kw["K"] % 2 == 0):
+            continue
+        try:
+            cfg = make_config(**kw)
+            v = kernelArgFromConfig(cfg).values()
+            if _native.is_valid_config(v, _native.KIND_MFMA) and \
+                    "DIRECT = true" in _native.instantiation_source(v, _native.KIND_MFMA):
+                if len(out) >= n and all(seen.get(c, 0) >= 6 for c in odd16_class(cfg)):
+                    continue
+                out.append((cfg, _native.KIND_MFMA))
+                for c in odd16_class(cfg):
+                    seen[c] = seen.get(c, 0) + 1
+        except (ValueError, _native.KcgError):
+            continue
+    return out
+
+
+def test_random_odd_16bit_shapes_through_the_direct_kernel_are_bit_exact():
+    """fp16 / bf16 with odd extents: every other row of an operand starts 2 bytes off a 4-byte boundary, the piece
+    at the end of a row brings the next row's first element with it, and the piece at the end of a matrix with an
+    even number of odd-length rows is fetched from 2 bytes further down and moved into place in LDS."""
+    cases = random_odd_16bit_direct_configs()
+    direct, classes = 0, {}
+    for i, (cfg, kind) in enumerate(cases):
+        M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+        lim = 2 if cfg["DATATYPE_C"] == 4 else 1       # 16-bit outputs: |sums| <= K <= 255 stay exact
+        a = SI.small_ints((M, K), SI.STREAM_A, lim=lim)
+        b = SI.small_ints((K, N), SI.STREAM_B, lim=lim)
+        print(f"[case] random odd 16-bit direct {i} {odd16_class(cfg)} {kernelArgFromConfig(cfg).values()}", flush=True)
+        got, info = run_gemm(cfg, a, b, kind)
+        if info["lds_bytes"] == 0:
+            direct += 1
+            for c in odd16_class(cfg):
+                classes[c] = classes.get(c, 0) + 1
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        bad = int((got.astype(np.float64) != want).sum()) + int(np.isnan(got).sum())
+        assert bad == 0, f"random odd 16-bit config {i} ({info['kernel_name']}): {bad} wrong elements"
+    # (configs whose per-lane fetch offsets do not fit the register file are built with register staging instead)
+    assert direct >= 28 and all(classes.get(c, 0) >= 4 for c in ("a-kcont", "a-rowcont", "b", "k-odd")), (direct, classes)
+
+
 def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
     cases = random_odd_direct_configs() + random_even_16bit_direct_configs()
     direct = 0
