@@ -240,8 +240,9 @@ bool mfma_direct(const MatmulConfig& c) {
   auto tile_ok = [g](int x) { return is_pow2(x) || (x > 0 && x % (16 * g) == 0); };
   if (!tile_ok(c.BM) || !tile_ok(c.BN) || !is_pow2(c.BK) || c.BM < 32 || c.BN < 32) return false;
   if ((c.BM * c.BK / g) % (64 * nw) || (c.BN * c.BK / g) % (64 * nw)) return false;
-  // (rows of A and B that do not start on 16-byte boundaries are fetched in 4-byte pieces: one fp32 element, or two
-  // 16-bit elements from an even column on, whatever the extents)
+  // (any K >= BK and any M and N that give A and B rows of at least one chunk: the 16-byte fetches take source
+  // addresses of any alignment)
+  if (c.N < g || (c.ATRANS ? c.M : c.K) < g) return false;
   const long lim = 1L << 31;                              // 32-bit byte offsets per lane inside a tile panel
   if ((long)c.BM * c.K * es >= lim || (long)c.BK * c.M * es >= lim || (long)c.BK * c.N * es >= lim) return false;
   return 2 * (c.BM + c.BN) * c.BK * es <= kMaxLdsBytes;

@@ -72,10 +72,13 @@ __device__ __forceinline__ unsigned long long tl_cycles() {
 // Family 2b: matrix-core kernel with direct global->LDS staging.
 //
 // Every lane fetches one 16-byte chunk (G = 4 fp32 or 8 fp16/bf16 elements) with
-// global_load_lds_dwordx4 (4 bytes with global_load_lds_dword where M, N or K is not a multiple of G, so that rows do
-// not start on 16-byte boundaries: one fp32 element, or two 16-bit ones when M, N and K are even); a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
+// global_load_lds_dwordx4; a wave's 64 chunks land in 1 KiB of consecutive LDS, so no register, no
 // ds_write and no vector ALU work is spent on staging, and with NST stages the fetch of a tile can be in
-// flight for NST-1 K tiles.  The LDS image keeps the orientation of global memory:
+// flight for NST-1 K tiles.  The source address of a chunk need not be 16-byte aligned: where M, N or K is
+// not a multiple of G the rows of A and B start anywhere (fp32: on 4-byte boundaries, fetched at the full
+// rate; 16-bit rows of odd length: every other one 2 bytes off, fetched at about 40 % of it), and the chunk
+// at the end of a row brings the first elements of the next row with it, which land in columns (or k values)
+// that do not exist and are never used.  The LDS image keeps the orientation of global memory:
 //   k-contiguous operand  (A, IS_ATRANS=0): rows = m, CH = BK/G chunks of G k values each; a fragment
 //                                           is one ds_read_b128 (as in gemm_mfma)
 //   row-contiguous operand (B; A^T)       : rows = k, NCH = BN/G (BM/G) chunks of G n values each.
@@ -150,29 +153,21 @@ struct DirectPlan {
   // block tile extents: a power of two, or a multiple of 16 chunks (the bank swizzle of a row-contiguous
   // tile exchanges chunks inside aligned groups of 16, so a row must consist of whole groups): 192, 320, ...
   static constexpr bool tile_ok(int x) { return pow2(x) || (x > 0 && x % (16 * G) == 0); }
-  // What a lane fetches: a whole 16-byte chunk where every row of A and B starts on a 16-byte boundary (M, N and K
-  // multiples of G); otherwise 4 bytes (the same instruction with a 4-byte payload: a wave's 64 pieces land in 256
-  // consecutive bytes of LDS) — one 4-byte element, or the two 2-byte elements at an even and the next odd column.
-  // With 16-bit rows of odd length every other row starts 2 bytes off a 4-byte boundary; the fetch takes such
-  // source addresses (at about 60 % of the aligned rate), and the piece at the end of a row brings the first
-  // element of the next row with it, which lands in a column (or k value) that does not exist and is never used.
-  static constexpr bool CHUNK_FETCH = C::M % G == 0 && C::N % G == 0 && C::K % G == 0;
-  static constexpr int FGMIN = ES <= 4 ? 4 / ES : 1;              // elements in 4 bytes
-  static constexpr bool PIECE_FETCH = ES <= 4;
-  static constexpr int FG = CHUNK_FETCH ? G : FGMIN;              // elements per lane and fetch instruction
-  // The piece that holds the last element of a matrix with odd rows would reach 2 bytes past the end of the buffer
-  // when it starts 2 bytes off a 4-byte boundary, i.e. when the matrix has an even number of rows; past the end may
-  // be another page.  Such a matrix gets its last piece from 2 bytes further down, and the lane that fetched it
-  // moves the element into place in LDS (see patch_final in the kernel).
-  static constexpr int A_ROWS = C::ATRANS ? C::K : C::M, A_COLS = C::ATRANS ? C::M : C::K;
-  static constexpr bool FIX_A = ES == 2 && A_COLS % 2 == 1 && A_ROWS % 2 == 0;
-  static constexpr bool FIX_B = ES == 2 && C::N % 2 == 1 && C::K % 2 == 0;
+  // The chunk at the end of the last row of a matrix whose rows are not whole chunks would reach up to 14 bytes
+  // past the end of the buffer, which may be another page.  It is fetched from SH_x elements further down
+  // instead (the last 16 bytes of the buffer), and the lane that fetched it moves the elements into place in LDS
+  // (patch_final in the kernel).
+  static constexpr int A_COLS = C::ATRANS ? C::M : C::K;          // row length of A as stored
+  static constexpr int SH_A = (G - A_COLS % G) % G, SH_B = (G - C::N % G) % G;
+  static constexpr bool FIX_A = SH_A != 0, FIX_B = SH_B != 0;
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
-      // edge tiles in M and N are fine; K needs one full tile
+      // edge tiles in M and N are fine; K needs one full tile, and a row of A or B as stored at least one chunk (with
+      // shorter rows several rows would share the chunk that reaches the end of the buffer)
+      C::N >= G && A_COLS >= G &&
       SPW > 0 && C::K >= C::BK && WM / MF >= 2 && tile_ok(C::BM) && tile_ok(C::BN) && pow2(C::BK) && C::BM >= 32 && C::BN >= 32 &&
-      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 && (CHUNK_FETCH || PIECE_FETCH) &&
+      (C::BM * C::BK / G) % (64 * NW) == 0 && (C::BN * C::BK / G) % (64 * NW) == 0 &&
       2 * (C::BM + C::BN) * C::BK * ES <= 160 * 1024 &&
       // fetch addresses are a scalar tile base + a 32-bit byte offset per lane
       (long)C::BM * C::K * ES < (1L << 31) && (long)C::BK * C::M * ES < (1L << 31) && (long)C::BK * C::N * ES < (1L << 31);
@@ -183,7 +178,7 @@ struct DirectPlan {
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
   // and no more than the fetch counter can tell apart: the wait for tile kt+1 allows the fetches of
   // NST-2 younger tiles in flight, and that counter has 6 bits
-  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / FG) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
+  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
   static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
   static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
   // Two blocks on a compute unit beat one block with deeper staging when the launch has more blocks than the
@@ -209,6 +204,83 @@ struct DirectPlan {
   static constexpr bool OK = C::DIRECT;
 };
 
+// Which 16 bytes of A and B the fetch instructions of a K tile bring to LDS: instruction idx of wave `wave` fills
+// the 64 consecutive chunk slots 64*(wave*NI + idx) .. +63 of the operand's stage, one per lane.  Host-callable: a
+// test walks every address of every tile of a problem through exactly this code.
+template <class C>
+struct FetchMap {
+  typedef DirectPlan<C> P;
+  static constexpr int ES = P::ES, G = P::G, NW = P::NW;
+  static constexpr int BM = C::BM, BN = C::BN, BK = C::BK, M = C::M, N = C::N, K = C::K;
+  static constexpr bool AK = !C::ATRANS;                          // A is k-contiguous in global memory
+  static constexpr bool EDGE_M = M % BM != 0, EDGE_N = N % BN != 0;
+  static constexpr int CHK = BK / G;                              // chunks per row of a k-contiguous tile
+  static constexpr int NCHA = BM / G, NCHB = BN / G;              // chunks per row of a row-contiguous tile
+  static constexpr int NIA = (BM * BK / G) / (64 * NW);           // fetch instructions per wave and tile, operand A
+  static constexpr int NIB = (BN * BK / G) / (64 * NW);
+  static constexpr int KT = K / BK;                               // full K tiles
+  static constexpr int KR = K % BK;                               // the remainder: one more, partial tile
+  static constexpr int KTT = KT + (KR > 0 ? 1 : 0);
+  // The last tile computes its fetch offsets on the spot instead of taking the registers all other tiles share
+  // when it is the partial one or holds a chunk that is fetched from another place (FIX_A / FIX_B).
+  // KTF: tiles in front of it; KLAST: its k extent.
+  static constexpr bool FINAL_SPECIAL = KR > 0 || P::FIX_A || P::FIX_B;
+  static constexpr int KTF = FINAL_SPECIAL ? KTT - 1 : KTT;
+  static constexpr int KLAST = KR > 0 ? KR : BK;
+  typedef LdsTile<CHK> LK;
+  // swizzle of a row-contiguous tile (chunk index ^= swz_n(row)).  16-bit: the rows that one pass of a
+  // transposing read touches (k..k+3, and k+8..k+11 with 16-wide matrix-core tiles) must not share banks.
+  // 32-bit: a fragment read is four 32-bit reads; in each, MF lanes read consecutive columns of one row
+  // and the 64/MF lane groups read rows 4 apart, which must fall into different bank ranges.
+  __host__ __device__ static constexpr int swz_n(int k, int nch) {
+    const int mask = nch >= 16 ? 15 : nch - 1;          // nch: a power of two below 16, or a multiple of 16
+    return (ES == 2 ? (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) : P::MF == 32 ? (((k >> 2) & 1) << 3) : (((k >> 2) & 3) << 2)) & mask;
+  }
+  // off: byte offset of the lane's chunk from the tile base.  moved: the chunk is the one at the end of the matrix and
+  // is fetched from SH elements further down (last_tile says that the tile is the last one of the K loop); only
+  // such a chunk can start in front of the tile base (off < 0).
+  struct Src {
+    int off;
+    bool moved;
+  };
+  // kvalid: how many k rows / values of the tile exist (BK, or KR for the partial tile)
+  __host__ __device__ static Src a(int wave, int lane, int idx, int m0, int kvalid, bool last_tile) {
+    const int s = 64 * (wave * NIA + idx) + lane;       // physical chunk slot inside the A stage
+    if constexpr (AK) {
+      int row = s / CHK;
+      const int cp = s % CHK;
+      int k = (cp ^ ((row / LK::RDIV) % LK::SMOD)) * G;
+      if constexpr (EDGE_M) row = cmin(row, M - 1 - m0);
+      if (k >= kvalid) k = 0;
+      const bool moved = P::FIX_A && last_tile && m0 + row == M - 1 && k + G > kvalid;
+      return Src{(row * K + k - (moved ? P::SH_A : 0)) * ES, moved};
+    } else {
+      int k = s / NCHA;
+      const int cp = s % NCHA;
+      int m = (cp ^ swz_n(k, NCHA)) * G;
+      if constexpr (EDGE_M) m = cmin(m, ((M - m0 - 1) / G) * G);   // the last chunk that starts inside the row
+      if (k >= kvalid) k = 0;
+      const bool moved = P::FIX_A && last_tile && k == kvalid - 1 && m0 + m + G > M;
+      return Src{(k * M + m - (moved ? P::SH_A : 0)) * ES, moved};
+    }
+  }
+  __host__ __device__ static Src b(int wave, int lane, int j, int n0, int kvalid, bool last_tile) {
+    const int s = 64 * (wave * NIB + j) + lane;
+    int k = s / NCHB;
+    const int cp = s % NCHB;
+    int n = (cp ^ swz_n(k, NCHB)) * G;
+    if constexpr (EDGE_N) n = cmin(n, ((N - n0 - 1) / G) * G);
+    if (k >= kvalid) k = 0;
+    const bool moved = P::FIX_B && last_tile && k == kvalid - 1 && n0 + n + G > N;
+    return Src{(k * N + n - (moved ? P::SH_B : 0)) * ES, moved};
+  }
+  // byte offset of a block's tile kt from the start of A / B
+  static constexpr long A_KT_BYTES = AK ? (long)BK * ES : (long)BK * M * ES;   // one K tile further
+  static constexpr long B_KT_BYTES = (long)BK * N * ES;
+  __host__ __device__ static constexpr long a_tile(int m0, int kt) { return (AK ? (long)m0 * K : (long)m0) * ES + kt * A_KT_BYTES; }
+  __host__ __device__ static constexpr long b_tile(int n0, int kt) { return (long)n0 * ES + kt * B_KT_BYTES; }
+};
+
 template <class C>
 __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restrict__ A, const typename C::TB* __restrict__ B,
                                                  typename C::TC* __restrict__ Cm, char* smem, EpiArgs ep = EpiArgs{1.f, 0.f}) {
@@ -220,25 +292,20 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int WM = P::WM, WN = P::WN, MF = P::MF;
   constexpr int KH = 64 / MF, KS = P::KS, SPW = P::SPW;
   constexpr int TMI = WM / MF, TNI = WN / MF, NM = P::NM, NW = P::NW;
-  constexpr int KT = K / BK;                            // full K tiles
-  constexpr int KR = K % BK, SPWT = cdiv(KR, KS);       // the remainder: one more tile of SPWT k-steps (the last may be partial)
-  constexpr int KTT = KT + (KR > 0 ? 1 : 0);
-  // The last tile computes its fetch offsets on the spot instead of taking the registers all other tiles share,
-  // when it is the partial one or holds a piece that is fetched from another place (FIX_A / FIX_B).
-  // KTF: tiles in front of it; KLAST: its k extent.
-  constexpr bool FINAL_SPECIAL = KR > 0 || P::FIX_A || P::FIX_B;
-  constexpr int KTF = FINAL_SPECIAL ? KTT - 1 : KTT;
-  constexpr int KLAST = KR > 0 ? KR : BK;
+  typedef FetchMap<C> FM;
+  constexpr int KT = FM::KT;                            // full K tiles
+  constexpr int KR = FM::KR, SPWT = cdiv(KR, KS);       // the remainder: one more tile of SPWT k-steps (the last may be partial)
+  constexpr int KTT = FM::KTT;
+  constexpr bool FINAL_SPECIAL = FM::FINAL_SPECIAL;     // the last tile computes its fetch offsets on the spot
+  constexpr int KTF = FM::KTF, KLAST = FM::KLAST;       // tiles in front of it; its k extent
   constexpr bool EDGE_M = M % BM != 0, EDGE_N = N % BN != 0;
   constexpr bool AK = !C::ATRANS;                       // A is k-contiguous in global memory
   constexpr int ES = P::ES, G = P::G;                   // element size; elements per 16-byte chunk
   constexpr int CHK = BK / G;                           // chunks per row of a k-contiguous tile
   constexpr int NCHA = BM / G, NCHB = BN / G;           // chunks per row of a row-contiguous tile
   constexpr int A_BYTES = BM * BK * ES, B_BYTES = BN * BK * ES, STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int FG = P::FG, GPC = G / FG;               // elements per lane and fetch; fetch granules per chunk
-  constexpr int NIA = (BM * BK / FG) / (64 * NW);       // fetch instructions per wave and tile, operand A
-  constexpr int NIB = (BN * BK / FG) / (64 * NW);
-  constexpr int FETCH_BYTES = 64 * FG * ES;             // LDS bytes one fetch instruction of a wave fills
+  constexpr int NIA = FM::NIA, NIB = FM::NIB;           // fetch instructions per wave and tile
+  constexpr int FETCH_BYTES = 64 * 16;                  // LDS bytes one fetch instruction of a wave fills
   typedef Mfma<T, MF> MI;
   typedef typename MI::Acc Acc;
   typedef typename MI::Frag Frag;
@@ -268,73 +335,21 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   (void)smem;
   auto stage_ptr = [&](auto stage_c) -> char* { return lds_all + decltype(stage_c)::value * STAGE_BYTES; };
 
-  // swizzle of a row-contiguous tile (chunk index ^= swz_n(row)).  16-bit: the rows that one pass of a
-  // transposing read touches (k..k+3, and k+8..k+11 with 16-wide matrix-core tiles) must not share banks.
-  // 32-bit: a fragment read is four 32-bit reads; in each, MF lanes read consecutive columns of one row
-  // and the 64/MF lane groups read rows 4 apart, which must fall into different bank ranges.
-  auto swz_n = [](int k, int nch) {
-    const int mask = nch >= 16 ? 15 : nch - 1;          // nch: a power of two below 16, or a multiple of 16
-    if constexpr (ES == 2) return (((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) & mask;
-    else if constexpr (MF == 32) return (((k >> 2) & 1) << 3) & mask;
-    else return (((k >> 2) & 3) << 2) & mask;
-  };
+  auto swz_n = [](int k, int nch) { return FM::swz_n(k, nch); };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
-  // never changes: the K loop spends no vector instruction on addresses.
-  // kvalid: how many k rows/values of the tile exist (BK, or KR for the partial tile)
-  // fix: the tile is the last one of the K loop and the piece with the matrix's last element is taken from 2 bytes
-  // further down (DirectPlan::FIX_A / FIX_B); *moved (optional) says whether this lane's piece is that one
-  auto off_a = [&](int idx, int kvalid, bool fix = false, bool* moved = nullptr) -> unsigned {
-    const int p = 64 * (wave * NIA + idx) + lane;     // physical fetch-granule slot inside the A stage
-    const int s = p / GPC, e = (p % GPC) * FG;        // chunk slot; first element of the granule inside its chunk
-    bool last = false;
-    unsigned off;
-    if constexpr (AK) {
-      int row = s / CHK;
-      const int cp = s % CHK;
-      const int c = cp ^ ((row / LK::RDIV) % LK::SMOD);
-      int k = c * G + e;
-      if constexpr (EDGE_M) row = cmin(row, M - 1 - m0);
-      last = P::FIX_A && fix && m0 + row == M - 1 && k == kvalid - 1;
-      if (k >= kvalid) k = 0;
-      off = (unsigned)((row * K + k) * ES);
-    } else {
-      int k = s / NCHA;
-      const int cp = s % NCHA;
-      const int c = cp ^ swz_n(k, NCHA);
-      int m = c * G + e;
-      if constexpr (EDGE_M) m = cmin(m, ((M - m0 - 1) / FG) * FG);   // the last piece that starts inside the row
-      last = P::FIX_A && fix && k == kvalid - 1 && m0 + m == M - 1;
-      if (k >= kvalid) k = 0;
-      off = (unsigned)((k * M + m) * ES);
-    }
-    if (moved) *moved = last;
-    return last ? off - ES : off;
-  };
-  auto off_b = [&](int j, int kvalid, bool fix = false, bool* moved = nullptr) -> unsigned {
-    const int p = 64 * (wave * NIB + j) + lane;
-    const int s = p / GPC, e = (p % GPC) * FG;
-    int k = s / NCHB;
-    const int cp = s % NCHB;
-    const int c = cp ^ swz_n(k, NCHB);
-    int n = c * G + e;
-    if constexpr (EDGE_N) n = cmin(n, ((N - n0 - 1) / FG) * FG);
-    const bool last = P::FIX_B && fix && k == kvalid - 1 && n0 + n == N - 1;
-    if (k >= kvalid) k = 0;
-    if (moved) *moved = last;
-    const unsigned off = (unsigned)((k * N + n) * ES);
-    return last ? off - ES : off;
-  };
+  // never changes (FetchMap): the K loop spends no vector instruction on addresses.
+  auto off_a = [&](int idx) -> unsigned { return (unsigned)FM::a(wave, lane, idx, m0, BK, false).off; };
+  auto off_b = [&](int j) -> unsigned { return (unsigned)FM::b(wave, lane, j, n0, BK, false).off; };
   unsigned voff_a[NIA], voff_b[NIB];
 #pragma unroll
-  for (int idx = 0; idx < NIA; ++idx) voff_a[idx] = off_a(idx, BK);
+  for (int idx = 0; idx < NIA; ++idx) voff_a[idx] = off_a(idx);
 #pragma unroll
-  for (int j = 0; j < NIB; ++j) voff_b[j] = off_b(j, BK);
-  const char* const a_base = (const char*)(AK ? A + (long)m0 * K : A + m0);
-  const char* const b_base = (const char*)(B + n0);
-  constexpr long A_KT_BYTES = AK ? (long)BK * ES : (long)BK * M * ES;   // one K tile further
-  constexpr long B_KT_BYTES = (long)BK * N * ES;
+  for (int j = 0; j < NIB; ++j) voff_b[j] = off_b(j);
+  const char* const a_base = (const char*)A + FM::a_tile(m0, 0);
+  const char* const b_base = (const char*)B + FM::b_tile(n0, 0);
+  constexpr long A_KT_BYTES = FM::A_KT_BYTES, B_KT_BYTES = FM::B_KT_BYTES;   // one K tile further
   // The tile bases pass through an empty asm: the compiler must not fold the per-tile scalar part
   // into the per-lane part (it would hoist "base + lane offset" as a 64-bit vector value and add the
   // tile offset with vector instructions); kept apart, the fetch uses its scalar-base addressing form.
@@ -350,60 +365,61 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     constexpr bool PARTIAL = decltype(partial_c)::value;
     char* st = stage_ptr(stage_c);
     if (idx < NIA) {
-      unsigned off;
-      if constexpr (PARTIAL) off = off_a(idx, KLAST, true);
+      long off;
+      if constexpr (PARTIAL) off = FM::a(wave, lane, idx, m0, KLAST, true).off;   // (signed: a moved chunk may start in front of the tile base)
       else {
         asm volatile("" : "+v"(voff_a[idx]));   // keeps the 32->64 bit extension next to the fetch (see tile_base)
-        off = voff_a[idx];
+        off = (long)(unsigned long)voff_a[idx];
       }
-      const char* src = tb.a + (unsigned long)off;
+      const char* src = tb.a + off;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + FETCH_BYTES * (wave * NIA + idx)), P::FG * P::ES, 0, KCG_FETCH_AUX);
+                                       (__attribute__((address_space(3))) void*)(st + FETCH_BYTES * (wave * NIA + idx)), 16, 0, KCG_FETCH_AUX);
     } else {
       const int j = idx - NIA;
-      unsigned off;
-      if constexpr (PARTIAL) off = off_b(j, KLAST, true);
+      long off;
+      if constexpr (PARTIAL) off = FM::b(wave, lane, j, n0, KLAST, true).off;
       else {
         asm volatile("" : "+v"(voff_b[j]));
-        off = voff_b[j];
+        off = (long)(unsigned long)voff_b[j];
       }
-      const char* src = tb.b + (unsigned long)off;
+      const char* src = tb.b + off;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + A_BYTES + FETCH_BYTES * (wave * NIB + j)), P::FG * P::ES, 0, KCG_FETCH_AUX);
+                                       (__attribute__((address_space(3))) void*)(st + A_BYTES + FETCH_BYTES * (wave * NIB + j)), 16, 0, KCG_FETCH_AUX);
     }
   };
   constexpr int NFETCH = NIA + NIB;
-  // FIX_A / FIX_B: the piece with the last element of the matrix was fetched from 2 bytes further down, so its
-  // 32-bit word in LDS holds the last element in the upper half.  The lane that fetched it shifts it down (what
-  // the upper half then stands for does not exist: a column beyond N, a row beyond M or a k value beyond K).
+  // FIX_A / FIX_B: the chunk at the end of the matrix was fetched from SH elements further down, so its 16 bytes in
+  // LDS hold the elements that exist in their upper part.  The lane that fetched it shifts them down (what the
+  // upper part then stands for does not exist: columns beyond N, rows beyond M or k values beyond K).
   // Called by every wave once its own fetches of the last tile have landed, in front of the barrier that
   // publishes the tile.
   auto patch_final = [&](auto stage_c) {
     const unsigned st = (unsigned)(unsigned long)stage_ptr(stage_c);
-    auto shift_down = [&](unsigned addr) {
-      unsigned w;
-      asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(w) : "v"(addr) : "memory");
-      w >>= 16;
-      asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(addr), "v"(w) : "memory");
+    auto shift_down = [&](unsigned addr, auto bytes_c) {
+      constexpr int SB = decltype(bytes_c)::value, WS = SB / 4, BS = (SB % 4) * 8;   // whole words; bits inside a word
+      u32x4 w;
+      asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(w) : "v"(addr) : "memory");
+      const unsigned in[8] = {w.x, w.y, w.z, w.w, 0u, 0u, 0u, 0u};
+      unsigned o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = BS ? (in[i + WS] >> BS) | (in[i + WS + 1] << ((32 - BS) % 32)) : in[i + WS];
+      w = u32x4{o[0], o[1], o[2], o[3]};
+      asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(addr), "v"(w) : "memory");
     };
     if constexpr (P::FIX_A) {
       if (m0 + BM >= M) {                       // (the block row with the last row of A, or its last column)
 #pragma unroll
-        for (int idx = 0; idx < NIA; ++idx) {
-          bool moved;
-          (void)off_a(idx, KLAST, true, &moved);
-          if (moved) shift_down(st + (unsigned)(FETCH_BYTES * (wave * NIA + idx) + lane * 4));
-        }
+        for (int idx = 0; idx < NIA; ++idx)
+          if (FM::a(wave, lane, idx, m0, KLAST, true).moved)
+            shift_down(st + (unsigned)(FETCH_BYTES * (wave * NIA + idx) + lane * 16), IntC<P::SH_A * ES>());
       }
     }
     if constexpr (P::FIX_B) {
       if (n0 + BN >= N) {
 #pragma unroll
-        for (int j = 0; j < NIB; ++j) {
-          bool moved;
-          (void)off_b(j, KLAST, true, &moved);
-          if (moved) shift_down(st + (unsigned)(A_BYTES + FETCH_BYTES * (wave * NIB + j) + lane * 4));
-        }
+        for (int j = 0; j < NIB; ++j)
+          if (FM::b(wave, lane, j, n0, KLAST, true).moved)
+            shift_down(st + (unsigned)(A_BYTES + FETCH_BYTES * (wave * NIB + j) + lane * 16), IntC<P::SH_B * ES>());
       }
     }
   };

@@ -119,7 +119,7 @@ template <int CH>
 struct LdsTile {
   static constexpr int SMOD = cmin(16, lowbit(CH));
   static constexpr int RDIV = cmax(1, 16 / SMOD);
-  __device__ __forceinline__ static int slot(int r, int c) { return r * CH + (c ^ ((r / RDIV) % SMOD)); }
+  __host__ __device__ __forceinline__ static int slot(int r, int c) { return r * CH + (c ^ ((r / RDIV) % SMOD)); }
 };
 
 }  // namespace kcg

@@ -1,0 +1,88 @@
+// kcg_fetch_check.h — host-side walk through the fetch map of the direct-staging kernel (FetchMap in
+// kcg_device_direct.h) for ONE instantiation: append this file to an instantiation stub (kcg_instantiation_source),
+// compile for the host and run.  For every block, K tile, wave, fetch instruction and lane it checks that
+//   * the 16 bytes fetched lie inside the operand's buffer (the kernel must never touch memory beyond A and B:
+//     what follows a buffer may be another page), and
+//   * every element of the tile that exists (row < M, column < N, k < K) ends up at the LDS position where the
+//     fragment reads look for it (LdsTile::slot for the k-contiguous operand, chunk ^ swz_n(row) for the
+//     row-contiguous ones), counting the shift that patch_final applies to a chunk fetched from further down.
+// Needs no GPU.  Prints one line and returns 0 when all is well.
+#pragma once
+#include <cstdio>
+
+int main() {
+  typedef kcg::DirectPlan<Cfg> P;
+  typedef kcg::FetchMap<Cfg> F;
+  if (!P::OK) {
+    printf("not a direct-staging instantiation\n");
+    return 2;
+  }
+  constexpr int M = F::M, N = F::N, K = F::K, BM = F::BM, BN = F::BN, BK = F::BK, G = F::G, ES = F::ES, NW = F::NW;
+  const long a_bytes = (long)M * K * ES, b_bytes = (long)K * N * ES;
+  const int gy = (M + BM - 1) / BM, gx = (N + BN - 1) / BN;
+  long chunks = 0, moved = 0, misaligned = 0;
+  // where the chunk in physical slot `phys` of an operand's stage comes from, after the shift of a moved chunk:
+  // the element index (in the operand's buffer) that LDS position i of the chunk holds is first + i for i < count
+  struct Got {
+    long first;
+    int count;
+  };
+  auto fail = [](const char* what, int by, int bx, int kt, int phys, long v) {
+    printf("FAILED: %s (block row %d, block column %d, K tile %d, chunk slot %d, value %ld)\n", what, by, bx, kt, phys, v);
+    return 1;
+  };
+  for (int by = 0; by < gy; ++by)
+    for (int bx = 0; bx < gx; ++bx) {
+      const int m0 = by * BM, n0 = bx * BN;
+      for (int kt = 0; kt < F::KTT; ++kt) {
+        const bool last = F::FINAL_SPECIAL && kt == F::KTF;
+        const int kvalid = last ? F::KLAST : BK;
+        auto fetched = [&](bool is_a, int phys, Got* g) -> int {
+          const int ni = is_a ? F::NIA : F::NIB;
+          const int wave = phys / (64 * ni), idx = (phys / 64) % ni, lane = phys % 64;
+          if (wave >= NW) return fail("chunk slot beyond the stage", by, bx, kt, phys, wave);
+          const typename F::Src s = is_a ? F::a(wave, lane, idx, m0, kvalid, last) : F::b(wave, lane, idx, n0, kvalid, last);
+          const long addr = (is_a ? F::a_tile(m0, kt) : F::b_tile(n0, kt)) + (long)s.off;
+          const long size = is_a ? a_bytes : b_bytes;
+          if (addr < 0 || addr + 16 > size) return fail(is_a ? "fetch outside A" : "fetch outside B", by, bx, kt, phys, addr);
+          if (addr % ES) return fail("fetch address not on an element boundary", by, bx, kt, phys, addr);
+          const int sh = s.moved ? (is_a ? P::SH_A : P::SH_B) : 0;
+          g->first = addr / ES + sh;
+          g->count = G - sh;
+          ++chunks;
+          moved += s.moved;
+          misaligned += (addr % 4) != 0;
+          return 0;
+        };
+        // A
+        for (int r = 0; r < (F::AK ? BM : BK); ++r)
+          for (int c = 0; c < (F::AK ? F::CHK : F::NCHA); ++c) {
+            const int phys = F::AK ? F::LK::slot(r, c) : r * F::NCHA + (c ^ F::swz_n(r, F::NCHA));
+            Got g;
+            if (fetched(true, phys, &g)) return 1;
+            for (int i = 0; i < G; ++i) {
+              const int row = F::AK ? m0 + r : m0 + c * G + i;            // m
+              const int kk = F::AK ? kt * BK + c * G + i : kt * BK + r;   // k
+              if (row >= M || row >= m0 + BM || kk >= K) continue;
+              const long want = F::AK ? (long)row * K + kk : (long)kk * M + row;
+              if (i >= g.count || g.first + i != want) return fail("A element not where the fragment reads look for it", by, bx, kt, phys, want);
+            }
+          }
+        // B
+        for (int r = 0; r < BK; ++r)
+          for (int c = 0; c < F::NCHB; ++c) {
+            const int phys = r * F::NCHB + (c ^ F::swz_n(r, F::NCHB));
+            Got g;
+            if (fetched(false, phys, &g)) return 1;
+            for (int i = 0; i < G; ++i) {
+              const int col = n0 + c * G + i, kk = kt * BK + r;
+              if (col >= N || kk >= K) continue;
+              const long want = (long)kk * N + col;
+              if (i >= g.count || g.first + i != want) return fail("B element not where the fragment reads look for it", by, bx, kt, phys, want);
+            }
+          }
+      }
+    }
+  printf("ok: %ld chunks, %ld fetched from further down, %ld from addresses off a 4-byte boundary\n", chunks, moved, misaligned);
+  return 0;
+}
