@@ -51,6 +51,14 @@ __device__ __forceinline__ void copy_bytes(void* dst, const void* src) {
   typedef typename RawVec<NBYTES>::type V;
   *reinterpret_cast<V*>(dst) = *reinterpret_cast<const V*>(src);
 }
+// The same where the addresses are aligned to ALIGN bytes only (ALIGN < NBYTES): still one access.  Global memory
+// takes vector accesses at element alignment; rows of C whose length is not a multiple of the vector are the case.
+template <int NBYTES, int ALIGN>
+__device__ __forceinline__ void copy_bytes_unaligned(void* dst, const void* src) {
+  typedef typename RawVec<NBYTES>::type V;
+  typedef V __attribute__((aligned(ALIGN))) VU;
+  *reinterpret_cast<VU*>(dst) = *reinterpret_cast<const VU*>(src);
+}
 // the same with a non-temporal store (streaming data that the kernel does not read again)
 template <int NBYTES>
 __device__ __forceinline__ void copy_bytes_nt(void* dst, const void* src) {
@@ -182,9 +190,15 @@ __device__ __forceinline__ void gstore(TC* __restrict__ base, const ACC* src, in
   } else if constexpr (ALIGNED) {
     if (r < RMAX && c < CMAX) copy_bytes<VEC * (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
   } else {
+    // a vector that lies inside the row goes out as one access at element alignment; the one across the end of
+    // the row element by element
+    if (VEC > 1 && r < RMAX && c + VEC <= CMAX) {
+      copy_bytes_unaligned<VEC * (int)sizeof(TC), (int)sizeof(TC)>(base + (long)r * LD + c, tmp);
+    } else {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e)
-      if (r < RMAX && c + e < CMAX) base[(long)r * LD + c + e] = tmp[e];
+      for (int e = 0; e < VEC; ++e)
+        if (r < RMAX && c + e < CMAX) base[(long)r * LD + c + e] = tmp[e];
+    }
   }
 }
 
