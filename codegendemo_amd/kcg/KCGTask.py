@@ -13,8 +13,9 @@ Counterpart of Runtime/python/kcg/KCGTask.py.  Control flow and file formats are
 
 What differs, on purpose: inputs are seeded (the reference draws unseeded torch.randn, :85-87), the
 timing loop runs in C with HIP events (kcg_benchmark) instead of one Python-level event pair per
-launch, and correctness is judged with the tolerance of the dtype (fp32: 1e-4*K*max|a|*max|b|;
-16-bit inputs: 2e-2 of the result scale) instead of allclose(atol=rtol=1e-1) (:177).
+launch, and correctness is judged with a tolerance that fits the dtype (fp32: 2e-6*K*max|a|*max|b|, a fiftieth of
+the acceptance bar of the parity tests, so that a kernel that drops one k-step is never ranked; 16-bit inputs: 2e-2
+of the result scale) instead of allclose(atol=rtol=1e-1) (:177).
 """
 import ctypes
 import glob

@@ -32,6 +32,9 @@ CASES = [
     ("f32-direct-edge-at1", MFMA, dict(M=200, N=136, K=104, BM=128, BN=64, TM=8, TN=4, BK=16, is_atrans=1, **DIRECT), 2),
     ("f16-direct", MFMA, dict(M=256, N=256, K=192, dtype=2, dtype_c=4, BM=128, BN=128, TM=8, TN=8, BK=64, is_atrans=0, **DIRECT), 2),
     ("bf16-mfma-at1", MFMA, dict(M=128, N=128, K=96, dtype=3, dtype_c=4, BM=64, BN=64, BK=32, is_atrans=1), 2),
+    # odd extents: rows off 4-byte boundaries, and the last chunk of every problem's A and B fetched from further down
+    ("f16-direct-odd", MFMA, dict(M=254, N=249, K=203, dtype=2, dtype_c=4, BM=128, BN=128, TM=8, TN=8, BK=64, is_atrans=0, **DIRECT), 3),
+    ("bf16-direct-odd-at1", MFMA, dict(M=125, N=131, K=128, dtype=3, dtype_c=4, BM=64, BN=64, TM=4, TN=4, BK=32, is_atrans=1, **DIRECT), 2),
 ]
 
 
@@ -92,7 +95,8 @@ def test_batched_alpha_beta_bit_exact_on_integers(oracle, tag, kind, kw, batch):
     M, N, K, at = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"], cfg["IS_ATRANS"]
     a = np.stack([SI.small_ints((M, K), 400 + z) for z in range(batch)])
     b = np.stack([SI.small_ints((K, N), 500 + z) for z in range(batch)])
-    sa, sb, sc = M * K + 16, K * N + 32, M * N + 8                 # padded strides (kept 16-byte aligned for every type)
+    pad8 = lambda x: (x + 7) // 8 * 8
+    sa, sb, sc = pad8(M * K) + 16, pad8(K * N) + 32, pad8(M * N) + 8   # padded strides (kept 16-byte aligned for every type)
     c0 = SI.small_ints((batch * sc,), 600).astype(np.float32)
     for alpha, beta in ((2.0, -3.0), (1.0, 1.0), (-0.5, 0.0)):
         print(f"[case] {tag} kind={kind} {M}x{N}x{K} batch={batch} alpha={alpha} beta={beta}", flush=True)
