@@ -287,6 +287,7 @@ def extra_build_configs():
     bf16["DATATYPE_A"] = bf16["DATATYPE_B"] = 3
     out.append((bf16, 0))
     out.append((SPILLING_FP64_CONFIG, MFMA))
+    out += [(make_config(*shape, **kw), MFMA) for _tag, shape, kw in LARGE_CASES]
     return out
 
 
@@ -295,6 +296,16 @@ def extra_build_configs():
 # build at the usual optimisation level returned wrong sums in the last block column
 SPILLING_FP64_CONFIG = dict(zip(_native.keywords(), [64, 64, 64, 4, 16, 64, 1, 1, 16, 4, 2, 2, 2, 2, 2, 2, 1, 4, 2, 4, 1, 1,
                                                       0, 1, 8, 8, 8, 8, 208, 592, 0]))
+
+# beyond the BASELINE sizes: eight times the work of config 3 / 5, extents that are no multiples of anything
+LARGE_CASES = (
+    ("fp16-8192", (8192, 8192, 8192), dict(dtype=2, dtype_c=4, BM=256, BN=256, TM=16, TN=16, BK=64, is_atrans=0, block_mapping=8,
+                                           shared_prefetch=1, reg_prefetch=1)),
+    ("bf16-odd-8191x8189x8195", (8191, 8189, 8195), dict(dtype=3, dtype_c=4, BM=256, BN=256, TM=16, TN=16, BK=32, is_atrans=0,
+                                                         block_mapping=8, shared_prefetch=1, reg_prefetch=1)),
+    ("fp32-odd-8190x8191x8193-at1", (8190, 8191, 8193), dict(BM=256, BN=256, TM=16, TN=8, BK=32, is_atrans=1,
+                                                             block_mapping=4, shared_prefetch=1, reg_prefetch=1)),
+)
 
 CONFIG4_KERNELS = ((MFMA, dict(BM=128, BN=128, TM=8, TN=8, BK=16, shared_prefetch=1, is_atrans=0)),
                    (MFMA, dict(BM=64, BN=64, BK=32, is_atrans=1)),
@@ -473,3 +484,34 @@ def test_kernel_that_needs_scratch_memory_is_exact(oracle):
     assert kernel.n_spills > 0
     kernel.unload()
     _exact_case(oracle, SPILLING_FP64_CONFIG, MFMA, "mfma-f64-one-wave-64x64x64-spilling")
+
+
+@pytest.mark.parametrize("tag,shape,kw", LARGE_CASES, ids=[c[0] for c in LARGE_CASES])
+def test_large_problems_are_exact_on_integers(oracle, tag, shape, kw):
+    """Problems of eight times the BASELINE work through the direct-staging kernel (row and tile offsets beyond
+    2^25 elements, 16 times the blocks of the tuned launch).  Operands are integers in [-2, 2] drawn on the device, so
+    every sum is exact in fp32 whatever the order: the whole result must equal the exact product bit for bit — taken
+    from an fp64 product on the device, which is exact as well (an independent route: the vendor library) — and a
+    row panel of it the CPU oracle's."""
+    import torch
+    from tests.gemm_helpers import build_kernel
+    M, N, K = shape
+    cfg = make_config(M, N, K, **kw)
+    kpm, ui, kernel, info = build_kernel(cfg, MFMA)
+    assert info["lds_bytes"] == 0, "expected the direct-staging kernel"
+    g = torch.Generator(device="cuda:0").manual_seed(20251127)
+    ta = kpm.dtypeTorch('A')
+    a = torch.randint(-2, 3, (M, K), device="cuda:0", generator=g).to(ta)
+    b = torch.randint(-2, 3, (K, N), device="cuda:0", generator=g).to(ta)
+    a_op = a.t().contiguous() if kpm.isATranspose else a
+    c = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda:0")
+    print(f"[case] large {tag} {M}x{N}x{K}", flush=True)
+    kernel.run(a_op, b, c)
+    torch.cuda.synchronize()
+    want = torch.matmul(a.to(torch.float64), b.to(torch.float64))
+    bad = int((c.to(torch.float64) != want).sum().item())          # NaN (never written) counts as different
+    assert bad == 0, f"{tag}: {bad} elements differ from the exact product"
+    rows = [0, 1, M // 2, M - 2, M - 1]
+    panel = oracle.matmul(a[rows].to(torch.float32).cpu().numpy(), b.to(torch.float32).cpu().numpy(), a_trans=False)
+    assert np.array_equal(c[rows].cpu().numpy(), panel)
+    kernel.unload()
