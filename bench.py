@@ -123,6 +123,23 @@ def time_steps(kernel, A, B, C, steps, warmup):
     return (t1 - t0) * 1e3 / steps, ev0.elapsed_time(ev1) / steps
 
 
+def reference_style_ms(kernel, A, B, C, samples=20):
+    """The reference's own measurement (KCGTask.py:124-130,164-171): one launch between a pair of events, host
+    synchronisation after every sample, median over the samples; includes what the launch costs from Python."""
+    import torch
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    ms = []
+    for _ in range(samples):
+        ev0.record()
+        kernel.run(A, B, C)
+        ev1.record()
+        torch.cuda.synchronize()
+        ms.append(ev0.elapsed_time(ev1))
+    ms.sort()
+    return 0.5 * (ms[(len(ms) - 1) // 2] + ms[len(ms) // 2])
+
+
 RAMP_LAUNCHES, STEADY_LAUNCHES = 100, 200
 
 
@@ -321,6 +338,7 @@ def main():
     value = flops / (ms_step * 1e-3) / 1e12
     achieved = flops / (ms_launch * 1e-3) / 1e12
     steady32 = steady_roofline(kernel, A, B, C, flops, PEAK_TFLOPS["f32"])
+    ref_ms = reference_style_ms(kernel, A, B, C)
     traffic32, traffic32_note = measured_traffic(info["kernel_name"])
 
     out = {
@@ -339,6 +357,8 @@ def main():
                      "launch_ms": ms_launch,
                      "hbm_gbs_algorithmic": (4.0 * (kpm.M * kpm.K + kpm.K * kpm.N + kpm.M * kpm.N)) / (ms_launch * 1e-3) / 1e9},
         "roofline_steady": steady32,
+        "reference_style_timing": {"ms": ref_ms, "tflops": flops / (ref_ms * 1e-3) / 1e12, "samples": 20,
+                                   "what": "one launch per event pair with a host synchronisation per sample, median (the reference's PerfTester)"},
     }
     for key, label, k_, kern_, info_, A_, B_, C_ in legs16:
         ms_step_, ms_launch_ = time_steps(kern_, A_, B_, C_, args.steps, args.warmup)
