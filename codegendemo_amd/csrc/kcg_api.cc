@@ -640,6 +640,7 @@ int kcg_launch(uint64_t function, const int32_t grid[3], const int32_t block[3],
   if (!function || !grid || !block) return fail(KCG_ERR_ARGUMENT, "null function / dims");
   if ((int64_t)grid[0] * grid[1] * grid[2] <= 0) return KCG_OK;  // empty grid: nothing to do
   if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
+  if ((a | b | c) & 15) return fail(KCG_ERR_ARGUMENT, "a, b and c must be 16-byte aligned");
   if (loaded_args(function) == 8) return fail(KCG_ERR_ARGUMENT, "this kernel has the batched-strided form: use kcg_launch_batched");
   void* pa = (void*)(uintptr_t)a;
   void* pb = (void*)(uintptr_t)b;
@@ -661,6 +662,7 @@ int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t b
   if ((int64_t)grid[0] * grid[1] * grid[2] <= 0 || batch == 0) return KCG_OK;  // nothing to do
   if (grid[1] != 1 || grid[2] != 1) return fail(KCG_ERR_ARGUMENT, "the batch goes on grid[1]: grid must be {n, 1, 1}");
   if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
+  if ((a | b | c) & 15) return fail(KCG_ERR_ARGUMENT, "a, b and c must be 16-byte aligned");
   if (loaded_args(function) == 3) return fail(KCG_ERR_ARGUMENT, "this kernel has the three-pointer form: use kcg_launch");
   void* pa = (void*)(uintptr_t)a;
   void* pb = (void*)(uintptr_t)b;

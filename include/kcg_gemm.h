@@ -169,7 +169,8 @@ int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int 
 
 /* hipModuleLaunchKernel(function, grid, block, lds_bytes, stream, {&a,&b,&c}); asynchronous on the
  * caller's stream (0 = null stream).  Skips the launch when the grid is empty (HIPLauncher.py:138).
- * a/b/c are device addresses owned by the caller.  A function that kcg_load handed out for a kernel of
+ * a/b/c are device addresses owned by the caller, 16-byte aligned (what hipMalloc and torch hand out: the kernels
+ * move 16-byte vectors; rows inside the matrices may start anywhere).  A function that kcg_load handed out for a kernel of
  * the batched-strided form (kcg_compile_matmul_ex) is refused with KCG_ERR_ARGUMENT: its parameter block
  * has eight entries (and kcg_launch_batched refuses a three-pointer kernel likewise). */
 int kcg_launch(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes,

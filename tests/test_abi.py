@@ -133,3 +133,12 @@ def test_register_staged_build_that_spills_is_rebuilt_at_a_lower_optimisation_le
     assert p_spill != p_spill_first and p_calm != p_calm_first          # the switch is part of the cache key
     assert code_spill != code_spill_first                               # the kept build is another one
     assert code_calm == code_calm_first                                 # nothing to rebuild
+
+
+def test_launch_refuses_misaligned_operand_addresses():
+    """The kernels move 16-byte vectors: an operand address that is not 16-byte aligned is refused before anything
+    is launched (the check comes before the first HIP call, so it can be seen without a GPU)."""
+    with pytest.raises(_native.KcgError, match="16-byte aligned"):
+        _native.launch(0x1000, [1, 1, 1], [64, 1, 1], 0, 0, 0x10000, 0x20004, 0x30000)
+    with pytest.raises(_native.KcgError, match="16-byte aligned"):
+        _native.launch_batched(0x1000, [1, 1, 1], [64, 1, 1], 0, 0, 0x10008, 0x20000, 0x30000, 2, 64, 64, 64)
