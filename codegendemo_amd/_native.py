@@ -51,6 +51,7 @@ EXPORTS = (
     "kcg_launch_dims", "kcg_reference_lds_bytes", "kcg_block_mapping", "kcg_compile_matmul",
     "kcg_instantiation_source", "kcg_load", "kcg_launch", "kcg_benchmark", "kcg_unload",
     "kcg_device_info", "kcg_last_error", "kcg_version", "kcg_compile_matmul_ex", "kcg_launch_batched",
+    "kcg_benchmark_batched",
 )
 
 _lib = None
@@ -125,6 +126,8 @@ def lib():
     L.kcg_launch_batched.argtypes = [ctypes.c_uint64, i32p, i32p, ctypes.c_int, ctypes.c_uint64,
                                      ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int32,
                                      ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_float, ctypes.c_float]
+    L.kcg_benchmark_batched.argtypes = L.kcg_launch_batched.argtypes + [ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                                        ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
     L.kcg_unload.argtypes = [ctypes.c_uint64]
     L.kcg_device_info.argtypes = [ctypes.c_int, i32p, i32p, i32p, ctypes.c_char_p, ctypes.c_int]
     _lib = L
@@ -257,6 +260,16 @@ def benchmark(function, grid, block, lds_bytes, stream, a, b, c, warmup=1, iters
     med, mn = ctypes.c_float(), ctypes.c_float()
     check(lib().kcg_benchmark(function, _dims(grid), _dims(block), int(lds_bytes), int(stream), int(a), int(b),
                               int(c), int(warmup), int(iters), int(reps), ctypes.byref(med), ctypes.byref(mn)))
+    return med.value, mn.value
+
+
+def benchmark_batched(function, grid, block, lds_bytes, stream, a, b, c, batch, stride_a, stride_b, stride_c, alpha=1.0, beta=0.0,
+                      warmup=1, iters=20, reps=0):
+    """-> (median_ms, min_ms) per launch of the whole batch"""
+    med, mn = ctypes.c_float(), ctypes.c_float()
+    check(lib().kcg_benchmark_batched(function, _dims(grid), _dims(block), int(lds_bytes), int(stream), int(a), int(b), int(c),
+                                      int(batch), int(stride_a), int(stride_b), int(stride_c), float(alpha), float(beta),
+                                      int(warmup), int(iters), int(reps), ctypes.byref(med), ctypes.byref(mn)))
     return med.value, mn.value
 
 

@@ -675,9 +675,10 @@ int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t b
   return KCG_OK;
 }
 
-int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes, uint64_t stream,
-                  uint64_t a, uint64_t b, uint64_t c, int warmup, int iters, int reps, float* median_ms,
-                  float* min_ms) {
+// The timing loop shared by kcg_benchmark and kcg_benchmark_batched: `launch` starts the kernel once on `stream`.
+extern "C++" {
+template <class Launch>
+static int timing_loop(uint64_t stream, int warmup, int iters, int reps, float* median_ms, float* min_ms, Launch launch) {
   if (iters <= 0) return fail(KCG_ERR_ARGUMENT, "iters must be positive");
   hipStream_t st = (hipStream_t)(uintptr_t)stream;
   hipEvent_t e0, e1;
@@ -696,7 +697,7 @@ int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[
     hipError_t e = HIPF(hipEventRecord)(e0, st);
     if (e != hipSuccess) return hip_fail(e, "hipEventRecord");
     for (int i = 0; i < n; ++i) {
-      int r = kcg_launch(function, grid, block, lds_bytes, stream, a, b, c);
+      int r = launch();
       if (r != KCG_OK) return r;
     }
     e = HIPF(hipEventRecord)(e1, st);
@@ -707,7 +708,7 @@ int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[
     if (e != hipSuccess) return hip_fail(e, "hipEventElapsedTime");
     return KCG_OK;
   };
-  for (int i = 0; i < warmup && rc == KCG_OK; ++i) rc = kcg_launch(function, grid, block, lds_bytes, stream, a, b, c);
+  for (int i = 0; i < warmup && rc == KCG_OK; ++i) rc = launch();
   if (rc == KCG_OK) {
     hipError_t e = HIPF(hipStreamSynchronize)(st);
     if (e != hipSuccess) rc = hip_fail(e, "hipStreamSynchronize");
@@ -733,6 +734,23 @@ int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[
   if (median_ms) *median_ms = (n % 2) ? samples[n / 2] : 0.5f * (samples[n / 2 - 1] + samples[n / 2]);
   if (min_ms) *min_ms = samples[0];
   return KCG_OK;
+}
+}  // extern "C++"
+
+int kcg_benchmark(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes, uint64_t stream,
+                  uint64_t a, uint64_t b, uint64_t c, int warmup, int iters, int reps, float* median_ms,
+                  float* min_ms) {
+  return timing_loop(stream, warmup, iters, reps, median_ms, min_ms,
+                     [&]() { return kcg_launch(function, grid, block, lds_bytes, stream, a, b, c); });
+}
+
+int kcg_benchmark_batched(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes, uint64_t stream,
+                          uint64_t a, uint64_t b, uint64_t c, int32_t batch, int64_t stride_a, int64_t stride_b,
+                          int64_t stride_c, float alpha, float beta, int warmup, int iters, int reps, float* median_ms,
+                          float* min_ms) {
+  return timing_loop(stream, warmup, iters, reps, median_ms, min_ms, [&]() {
+    return kcg_launch_batched(function, grid, block, lds_bytes, stream, a, b, c, batch, stride_a, stride_b, stride_c, alpha, beta);
+  });
 }
 
 int kcg_unload(uint64_t module) {

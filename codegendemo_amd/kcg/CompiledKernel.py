@@ -52,5 +52,10 @@ class CompiledKernel:
         """HIP-event timing in C: (median_ms, min_ms) per launch."""
         return self.m_launcher.benchmarkKernel(self.device, a, b, c, warmup, iters, reps)
 
+    def benchmark_batched(self, a, b, c, batch, stride_a, stride_b, stride_c, alpha=1.0, beta=0.0, warmup=1, iters=20, reps=0):
+        """HIP-event timing in C of the batched launch: (median_ms, min_ms) per batch."""
+        return self.m_launcher.benchmarkKernelBatched(self.device, a, b, c, batch, stride_a, stride_b, stride_c, alpha, beta,
+                                                      warmup, iters, reps)
+
     def unload(self):
         self.m_loader.unloadBinary(self.m_launcher.m_kernelLib)

@@ -74,3 +74,15 @@ class HIPLauncher:
         a, b, c = (_device_address(x) for x in (a, b, c))
         return _native.benchmark(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,
                                  DeviceInfo.get_cuda_stream(devId), a, b, c, warmup, iters, reps)
+
+    def benchmarkKernelBatched(self, devId: int, a, b, c, batch, stride_a, stride_b, stride_c, alpha=1.0, beta=0.0,
+                               warmup=1, iters=20, reps=0):
+        """The same timing loop around the batched launch (kcg_benchmark_batched): (median_ms, min_ms) per batch."""
+        if not self.m_kernelLib.m_kernelFuncName.endswith(("EX_", "EXab_")):
+            raise TypeError("this kernel was not compiled in the batched-strided form (KCGCompiler(epilogue=...))")
+        self._check_operands((a, b, c), batch, (stride_a, stride_b, stride_c))
+        fn = self._function()
+        a, b, c = (_device_address(x) for x in (a, b, c))
+        return _native.benchmark_batched(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,
+                                         DeviceInfo.get_cuda_stream(devId), a, b, c, batch, stride_a, stride_b, stride_c,
+                                         alpha, beta, warmup, iters, reps)

@@ -155,6 +155,13 @@ int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t b
                        uint64_t stream, uint64_t a, uint64_t b, uint64_t c, int32_t batch,
                        int64_t stride_a, int64_t stride_b, int64_t stride_c, float alpha, float beta);
 
+/* kcg_benchmark for a kernel of the batched-strided form: the same timing loop around kcg_launch_batched (one
+ * launch = the whole batch).  With beta != 0 every launch reads what the previous one wrote to C. */
+int kcg_benchmark_batched(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes,
+                          uint64_t stream, uint64_t a, uint64_t b, uint64_t c, int32_t batch,
+                          int64_t stride_a, int64_t stride_b, int64_t stride_c, float alpha, float beta,
+                          int warmup, int iters, int reps, float* median_ms, float* min_ms);
+
 /* The HIP source text that kcg_compile_matmul would hand to hiprtc for this config (the generated
  * instantiation stub; the template header is embedded in the library).  Returns bytes needed. */
 int kcg_instantiation_source(const kcg_matmul_cfg* cfg, int kind, char* out, int out_len);

@@ -183,3 +183,28 @@ def test_launch_batched_argument_checks():
         _native.launch_batched(fn, ui.m_gridDims, ui.m_blockDims, ui.m_shmSize, 0, a.data_ptr(), b.data_ptr(), c.data_ptr(),
                                1, 0, 0, 0)
     plain.unload()
+
+
+def test_batched_benchmark_times_the_whole_batch(oracle):
+    """kcg_benchmark_batched: the C timing loop around the batched launch; C afterwards is the batch's result."""
+    import torch
+    tag, kind, kw, batch = CASES[8]
+    cfg = make_config(**kw)
+    M, N, K = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"]
+    kpm, kernel, info = build(cfg, kind, AB)
+    a = np.stack([SI.small_ints((M, K), 1000 + z) for z in range(batch)])
+    b = np.stack([SI.small_ints((K, N), 1100 + z) for z in range(batch)])
+    a_dev = to_device(a.reshape(-1), kpm.dtypeTorch('A'))
+    b_dev = to_device(b.reshape(-1), kpm.dtypeTorch('A'))
+    c_dev = torch.full((batch * M * N,), float("nan"), dtype=torch.float32, device="cuda:0")
+    print(f"[case] batched benchmark {tag} {M}x{N}x{K} batch={batch}", flush=True)
+    med, mn = kernel.benchmark_batched(a_dev, b_dev, c_dev, batch, M * K, K * N, M * N, alpha=2.0, beta=0.0, warmup=2, iters=5, reps=3)
+    torch.cuda.synchronize()
+    assert 0 < mn <= med < 100.0
+    got = c_dev.cpu().numpy().reshape(batch, M, N)
+    for z in range(batch):
+        assert np.array_equal(got[z], 2.0 * oracle.matmul(a[z], b[z], a_trans=False))
+    kernel.unload()
+    plain = build(make_config(M=128, N=192, K=64), SIMT, None)[1]          # a three-pointer kernel
+    with pytest.raises(TypeError):
+        plain.benchmark_batched(a_dev, b_dev, c_dev, 1, 0, 0, 0)
