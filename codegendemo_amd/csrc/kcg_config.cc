@@ -84,7 +84,10 @@ static std::string fmt(const char* what, int a) {
 
 std::string check_common(const MatmulConfig& c) {
   if (c.M <= 0 || c.N <= 0 || c.K <= 0) return "M_SIZE, N_SIZE, K_SIZE must be positive";
+  // (the kernels index rows, columns and blocks with 32-bit integers; element offsets are 64-bit)
+  if (c.M > (1 << 30) || c.N > (1 << 30) || c.K > (1 << 30)) return "M_SIZE, N_SIZE, K_SIZE must not exceed 2^30";
   if (c.BM <= 0 || c.BN <= 0 || c.BK <= 0) return "BLOCK_SIZE_M/N/K must be positive";
+  if ((long)((c.M + c.BM - 1) / c.BM) * ((c.N + c.BN - 1) / c.BN) > 0x7fffffffL) return "more than 2^31 - 1 blocks";
   if (c.TM <= 0 || c.TN <= 0) return "THREAD_SIZE_M/N must be positive";
   if (c.WARP_SIZE != 64) return fmt("WARP_SIZE must be 64 on gfx950", c.WARP_SIZE);
   if (c.BLM <= 0 || c.BLN <= 0 || c.WLM <= 0 || c.WLN <= 0) return "BLOCK_LAYOUT / WARP_LAYOUT must be positive";

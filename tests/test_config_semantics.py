@@ -155,6 +155,8 @@ def test_invalid_configs_are_reported_not_compiled():
         "GLOB_LOAD_WIDTH": dict(good, GLOB_LOAD_WIDTH_A=0),
         "DATATYPE": dict(good, DATATYPE_A=2),                              # A != B
         "positive": dict(good, K_SIZE=0),
+        "2^30": dict(good, M_SIZE=2**31 - 1),                               # rows are indexed with 32-bit integers
+        "blocks": dict(good, M_SIZE=2**30, N_SIZE=2**30),
         "1024": dict(make_config(1024, 1024, 1024, BM=256, BN=256, BK=16, TM=8, TN=8), LOCAL_SPLIT_U=2),
     }
     for needle, cfg in cases.items():
