@@ -152,8 +152,7 @@ __device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r,
     if constexpr (ALIGNED) {
       copy_bytes<VEC * (int)sizeof(T)>(dst, base + (long)r * LD + c);
     } else {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) dst[e] = base[(long)r * LD + c + e];
+      copy_bytes_unaligned<VEC * (int)sizeof(T), (int)sizeof(T)>(dst, base + (long)r * LD + c);
     }
   } else if constexpr (ALIGNED) {
     // c and CMAX are multiples of VEC: the vector lies inside or outside as a whole.  No branch: a lane
@@ -162,12 +161,22 @@ __device__ __forceinline__ void gload(T* dst, const T* __restrict__ base, int r,
     copy_bytes<VEC * (int)sizeof(T)>(dst, base + (in ? (long)r * LD + c : 0L));
 #pragma unroll
     for (int e = 0; e < VEC; ++e) dst[e] = in ? dst[e] : T(0);
+  } else if constexpr (VEC == 1) {
+    const bool in = r < RMAX && c < CMAX;
+    const T v = base[in ? (long)r * LD + c : 0L];
+    dst[0] = in ? v : T(0);
   } else {
+    // rows that do not start on vector boundaries: a vector that lies inside its row is still one access (at element
+    // alignment, branch-free like the aligned case); only the vector across the end of a row goes element by element
+    const bool whole = r < RMAX && c + VEC <= CMAX;
+    copy_bytes_unaligned<VEC * (int)sizeof(T), (int)sizeof(T)>(dst, base + (whole ? (long)r * LD + c : 0L));
+    if (!whole) {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      const bool in = r < RMAX && c + e < CMAX;
-      const T v = base[in ? (long)r * LD + c + e : 0L];
-      dst[e] = in ? v : T(0);
+      for (int e = 0; e < VEC; ++e) {
+        const bool in = r < RMAX && c + e < CMAX;
+        const T v = base[in ? (long)r * LD + c + e : 0L];
+        dst[e] = in ? v : T(0);
+      }
     }
   }
 }
