@@ -192,7 +192,7 @@ def test_instantiation_source_carries_the_config():
 @pytest.mark.parametrize("shape,kw,direct", [
     ((4096, 1536, 1000), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # K = 62*16 + 8: one k-step of 8 left over
     ((4096, 1536, 1004), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # remainder 12: a whole k-step and half of one
-    ((4096, 1536, 1002), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # fp32, K not a multiple of the 16-byte vector: element-granular fetch
+    ((4096, 1536, 1002), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # fp32, K not a multiple of the 16-byte vector: rows off 16-byte boundaries
     ((4095, 1533, 1001), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),      # fp32, odd in every dimension
     ((4096, 1536, 8), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),        # not even one full K tile
     ((200, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),         # rows and columns beyond M and N
@@ -203,7 +203,7 @@ def test_instantiation_source_carries_the_config():
     ((256, 256, 1008), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # remainder 48 = 1.5 k-steps
     ((256, 256, 1004), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, K % 8 != 0 but even: two elements per lane
     ((256, 256, 1003), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, K odd: every other row of A starts 2 bytes off a 4-byte boundary
-    ((256, 255, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, N odd and K even: the last piece of B is fetched from 2 bytes further down
+    ((256, 255, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, N odd: the last chunk of B is fetched from further down
     ((256, 256, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4, load_continuous=0), False),
     ((1024, 1024, 1024), dict(BM=32, BN=32, BK=16, TM=4, TN=4, is_atrans=1), True),        # one wave, 2x2 tiles of 16x16
     ((1024, 1024, 1024), dict(BM=32, BN=64, BK=16, TM=2, TN=8, warp_layout=(8, 8)), False),  # 16-row wave tile: one row of tiles

@@ -193,9 +193,11 @@ def random_even_16bit_direct_configs(n=20, seed=20251126):
 
 
 def odd16_class(cfg):
-    """Which special case of 16-bit rows of odd length a config exercises: 'a-kcont' / 'a-rowcont' / 'b' — the last
-    piece of that operand would reach past the buffer and is fetched from 2 bytes further down; 'k-odd' — the last
-    k value shares its 32-bit word with one that does not exist; 'plain' — odd rows, none of these."""
+    """Which special case of 16-bit rows of odd length a config exercises: 'a-kcont' / 'a-rowcont' / 'b' — that operand
+    has an even number of odd-length rows, so its last row starts 2 bytes off a 4-byte boundary (the chunk at its end is
+    fetched from further down and shifted into place, like the last chunk of every matrix whose rows are not whole
+    chunks); 'k-odd' — the last k value shares its 32-bit word with one that does not exist; 'plain' — odd rows, none
+    of these."""
     M, N, K, at = cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"], cfg["IS_ATRANS"]
     out = []
     if not at and K % 2 == 1 and M % 2 == 0:
@@ -245,9 +247,9 @@ def random_odd_16bit_direct_configs(n=36, seed=20251127):
 
 
 def test_random_odd_16bit_shapes_through_the_direct_kernel_are_bit_exact():
-    """fp16 / bf16 with odd extents: every other row of an operand starts 2 bytes off a 4-byte boundary, the piece
-    at the end of a row brings the next row's first element with it, and the piece at the end of a matrix with an
-    even number of odd-length rows is fetched from 2 bytes further down and moved into place in LDS."""
+    """fp16 / bf16 with odd extents: every other row of an operand starts 2 bytes off a 4-byte boundary, the chunk
+    at the end of a row brings the next row's first elements with it, and the chunk at the end of the matrix is fetched
+    from further down and moved into place in LDS."""
     cases = random_odd_16bit_direct_configs()
     direct, classes = 0, {}
     for i, (cfg, kind) in enumerate(cases):
