@@ -197,11 +197,11 @@ def test_instantiation_source_carries_the_config():
     ((4096, 1536, 8), dict(BM=128, BN=64, BK=16, TM=8, TN=4), False),        # not even one full K tile
     ((200, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),         # rows and columns beyond M and N
     ((202, 136, 104), dict(BM=128, BN=64, BK=16, TM=8, TN=4), True),         # fp32, M not a multiple of the 16-byte vector
-    ((256, 252, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=3, dtype_c=4), True),   # bf16, N % 8 != 0 but even
+    ((256, 252, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=3, dtype_c=4), True),   # bf16, N % 8 != 0: rows of B off 16-byte boundaries
     ((255, 252, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=3, dtype_c=4), True),   # bf16, M odd (A's row count: nothing changes for the fetch)
     ((256, 256, 992), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),    # 16x16x32 tiles: k-steps of 32
     ((256, 256, 1008), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # remainder 48 = 1.5 k-steps
-    ((256, 256, 1004), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, K % 8 != 0 but even: two elements per lane
+    ((256, 256, 1004), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, K % 8 != 0: rows of A off 16-byte boundaries
     ((256, 256, 1003), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, K odd: every other row of A starts 2 bytes off a 4-byte boundary
     ((256, 255, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4), True),   # fp16, N odd: the last chunk of B is fetched from further down
     ((256, 256, 1024), dict(BM=128, BN=128, BK=64, TM=8, TN=8, dtype=2, dtype_c=4, load_continuous=0), False),
