@@ -327,9 +327,15 @@ def main():
         cfg16 = load_tuned(args.fp16_config or "gemm_4096_fp16.json")
         cfgb = dict(cfg16)
         cfgb["DATATYPE_A"] = cfgb["DATATYPE_B"] = 3      # the same config with bfloat16 inputs
-        for key, label, cfg in (("fp16", "f16", cfg16), ("bf16", "bf16", cfgb)):
+        cfgh = dict(cfg16)
+        cfgh["DATATYPE_C"] = 2                           # ... and with fp16 output (what the library's fp16 GEMM returns)
+        for key, label, cfg in (("fp16", "f16", cfg16), ("bf16", "bf16", cfgb), ("fp16_out16", "f16", cfgh)):
             k_, kern_, info_ = build_kernel(cfg)
-            _, _, A_, B_, C_ = make_inputs(k_, "normal")
+            if key == "fp16_out16":                      # the fp16 leg's operands, a result buffer of its own
+                A_, B_ = legs16[0][5], legs16[0][6]
+                C_ = torch.zeros((k_.M, k_.N), dtype=k_.dtypeTorch('C'), device="cuda:0")
+            else:
+                _, _, A_, B_, C_ = make_inputs(k_, "normal")
             legs16.append((key, label, k_, kern_, info_, A_, B_, C_))
     torch.cuda.synchronize()
 
@@ -365,7 +371,8 @@ def main():
         ach_ = flops / (ms_launch_ * 1e-3) / 1e12
         traffic_, traffic_note_ = measured_traffic(info_["kernel_name"])
         out[key] = {"value": flops / (ms_step_ * 1e-3) / 1e12, "unit": "TFLOPS", "ms_per_step": ms_step_,
-                    "dtype": f"{label} in, f32 accumulate/out", "kernel": info_["kernel_name"],
+                    "dtype": f"{label} in, f32 accumulate/out" if k_.dtypeTorch('C') == torch.float32 else f"{label} in, f32 accumulate, {label} out",
+                    "kernel": info_["kernel_name"],
                     "roofline": {"bound": "mfma", "achieved": ach_, "peak": PEAK_TFLOPS[label], "unit": "TFLOP/s",
                                  "frac": ach_ / PEAK_TFLOPS[label], "traffic": traffic_, "traffic_source": traffic_note_,
                                  "launch_ms": ms_launch_},
@@ -379,7 +386,8 @@ def main():
         _, _, k_, _, _, A_, B_, _ = legs16[0]
         lib16_ms = time_library_gemm(A_, B_, k_.isATranspose, args.steps, args.warmup)
         out["library_gemm"]["f16_tflops"] = flops / (lib16_ms * 1e-3) / 1e12
-        out["library_gemm"]["f16_note"] = "torch.matmul on fp16 operands returns fp16: the library writes 32 MiB of C, this engine 64 MiB of fp32"
+        out["library_gemm"]["f16_note"] = ("torch.matmul on fp16 operands returns fp16: the library writes 32 MiB of C, this engine's fp16 leg 64 MiB "
+                                           "of fp32 (BASELINE config 5); its fp16_out16 leg is the like-for-like figure")
 
     # ---- checks and side information (nothing below is timed)
     if not args.no_cpu:     # (skipped in profiling runs, like the CPU leg)
