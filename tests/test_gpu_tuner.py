@@ -62,6 +62,31 @@ def test_perf_tester_fp16_in_process(tmp_path, monkeypatch):
     PerfTester.torch_eps = 0.0
 
 
+ODD_BF16_CONFIG = make_config(1023, 1021, 1027, dtype=3, dtype_c=4, BM=128, BN=128, BK=32, TM=8, TN=8, is_atrans=1,
+                              shared_prefetch=1, reg_prefetch=1)
+
+
+def test_perf_tester_odd_extents_bf16_in_process(tmp_path, monkeypatch):
+    """The tuner's own measurement and correctness gate on a problem the reference's checker rejects outright
+    (matmul.py:293-298 wants M, N, K divisible by the tile): odd M, N and K, bf16, the `[K,M]` A layout."""
+    monkeypatch.setenv("KCG_WORK_DIR", str(tmp_path / "work"))
+    PathManager.init(clearCache=True)
+    from tests.gemm_helpers import build_kernel
+    PerfTester._a = PerfTester._b = None
+    PerfTester.torch_eps = 0.0
+    PerfTester.D = None
+    print("[case] PerfTester bf16 1023x1021x1027", flush=True)
+    kpm, ui, kernel, info = build_kernel(ODD_BF16_CONFIG)
+    assert info["lds_bytes"] == 0                   # the direct-staging path
+    PerfTester.setDevice(0)
+    PerfTester._init_AB(kpm, ui)
+    r = PerfTester._test_perf(kpm, ui, kernel, benchmarkCount=5, warmupCount=1, nTorchEpsInitTest=5)
+    assert r.isCorrect and r.tflops > 10 and r.acc > 0
+    PerfTester._a = PerfTester._b = PerfTester._aT = None
+    PerfTester.D = None
+    PerfTester.torch_eps = 0.0
+
+
 @pytest.mark.parametrize("case", ["case_normal_0", "case_normal_1"])
 def test_single_config_check_script(case, capsys):
     """python -m codegendemo_amd.kcg.test <case>: compile, one run, allclose(1e-2) against torch.matmul."""
