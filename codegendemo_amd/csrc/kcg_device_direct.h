@@ -809,7 +809,21 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
         // (N a multiple of 4: every group of four columns is one aligned 16-byte vector, inside or outside as a whole)
         if constexpr (C::EPI) epi_apply<TC, float, 4, (EDGE_M || EDGE_N), (N % 4 == 0)>(v, Cm, row, col, N, M, N, ep);
+#if defined(KCG_DIAG_STORE_LINES)
+        // diagnostic build (C WRONG: values land in other places): the same 64 store instructions per wave, each writing
+        // KCG_DIAG_STORE_LINES*64 contiguous bytes per row (2: whole 128-byte lines of 8 rows, 4: 256 bytes of 4 rows)
+        // instead of 64 bytes of 16 rows
+        {
+          constexpr int LPR = 4 * KCG_DIAG_STORE_LINES, RPI = 64 / LPR;      // lanes per row; rows per instruction
+          const int t = (i * TNI + j) * (NACC / 4) + g;
+          constexpr int CG = WN / (LPR * 4);                                  // column groups per wave tile
+          const int drow = m0 + wy * WM + (t / CG) * RPI + lane % RPI;
+          const int dcol = n0 + wx * WN + (t % CG) * (LPR * 4) + (lane / RPI) * 4;
+          gstore<TC, float, 4, (EDGE_M || EDGE_N), (N % 4 == 0), (KCG_C_NT != 0)>(Cm, v, drow, dcol, N, M, N);
+        }
+#else
         gstore<TC, float, 4, (EDGE_M || EDGE_N), (N % 4 == 0), (KCG_C_NT != 0)>(Cm, v, row, col, N, M, N);
+#endif
       }
 #if KCG_TIMELINE
   asm volatile("" ::: "memory");
