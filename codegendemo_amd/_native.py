@@ -43,7 +43,16 @@ class KernelInfo(ctypes.Structure):
         ("lds_bytes", ctypes.c_int32),
         ("kind", ctypes.c_int32),
         ("cache_hit", ctypes.c_int32),
+        ("build_flags", ctypes.c_int32),
+        ("scratch_bytes", ctypes.c_int32),
+        ("vgprs", ctypes.c_int32),
+        ("sgpr_spills", ctypes.c_int32),
     ]
+
+
+# kcg_build_flag bits
+BUILD_LOW_OPT, BUILD_DIAGNOSTIC, BUILD_DIRECT_DECLINED, BUILD_META_UNKNOWN = 1, 2, 4, 8
+SYSTEM_HIPRTC = "/opt/rocm/lib/libhiprtc.so.7"
 
 
 EXPORTS = (
@@ -51,7 +60,7 @@ EXPORTS = (
     "kcg_launch_dims", "kcg_reference_lds_bytes", "kcg_block_mapping", "kcg_compile_matmul",
     "kcg_instantiation_source", "kcg_load", "kcg_launch", "kcg_benchmark", "kcg_unload",
     "kcg_device_info", "kcg_last_error", "kcg_version", "kcg_compile_matmul_ex", "kcg_launch_batched",
-    "kcg_benchmark_batched",
+    "kcg_benchmark_batched", "kcg_code_object_info", "kcg_compiler_identity",
 )
 
 _lib = None
@@ -128,6 +137,8 @@ def lib():
                                      ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_float, ctypes.c_float]
     L.kcg_benchmark_batched.argtypes = L.kcg_launch_batched.argtypes + [ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                                         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
+    L.kcg_code_object_info.argtypes = [ctypes.c_char_p, ctypes.POINTER(KernelInfo)]
+    L.kcg_compiler_identity.argtypes = [ctypes.c_char_p, ctypes.c_int]
     L.kcg_unload.argtypes = [ctypes.c_uint64]
     L.kcg_device_info.argtypes = [ctypes.c_int, i32p, i32p, i32p, ctypes.c_char_p, ctypes.c_int]
     _lib = L
@@ -217,16 +228,7 @@ def instantiation_source(values, kind=KIND_AUTO):
     return buf.value.decode()
 
 
-def compile_matmul(values, arch="gfx950", kind=KIND_AUTO, epilogue=None):
-    """-> dict(code_path, kernel_name, grid, block, lds_bytes, kind, cache_hit).
-    epilogue None: the reference's three-pointer kernel; EPILOGUE_NONE / EPILOGUE_ALPHA_BETA: the
-    batched-strided kernel form (launch it with launch_batched)."""
-    c = make_cfg(values)
-    info = KernelInfo()
-    if epilogue is None:
-        check(lib().kcg_compile_matmul(ctypes.byref(c), arch.encode(), kind, ctypes.byref(info)))
-    else:
-        check(lib().kcg_compile_matmul_ex(ctypes.byref(c), arch.encode(), kind, int(epilogue), ctypes.byref(info)))
+def _info_dict(info):
     return {
         "code_path": info.code_path.decode(),
         "kernel_name": info.kernel_name.decode(),
@@ -235,7 +237,69 @@ def compile_matmul(values, arch="gfx950", kind=KIND_AUTO, epilogue=None):
         "lds_bytes": info.lds_bytes,
         "kind": info.kind,
         "cache_hit": bool(info.cache_hit),
+        "build_flags": info.build_flags,
+        "low_opt": bool(info.build_flags & BUILD_LOW_OPT),
+        "diagnostic": bool(info.build_flags & BUILD_DIAGNOSTIC),
+        "direct_declined": bool(info.build_flags & BUILD_DIRECT_DECLINED),
+        "scratch_bytes": info.scratch_bytes,
+        "vgprs": info.vgprs,
+        "sgpr_spills": info.sgpr_spills,
     }
+
+
+def compile_matmul(values, arch="gfx950", kind=KIND_AUTO, epilogue=None):
+    """-> dict(code_path, kernel_name, grid, block, lds_bytes, kind, cache_hit, build_flags, low_opt, diagnostic,
+    direct_declined, scratch_bytes, vgprs, sgpr_spills).
+    epilogue None: the reference's three-pointer kernel; EPILOGUE_NONE / EPILOGUE_ALPHA_BETA: the
+    batched-strided kernel form (launch it with launch_batched)."""
+    c = make_cfg(values)
+    info = KernelInfo()
+    if epilogue is None:
+        check(lib().kcg_compile_matmul(ctypes.byref(c), arch.encode(), kind, ctypes.byref(info)))
+    else:
+        check(lib().kcg_compile_matmul_ex(ctypes.byref(c), arch.encode(), kind, int(epilogue), ctypes.byref(info)))
+    return _info_dict(info)
+
+
+def code_object_info(code_path):
+    """What the compile recorded beside a code object it wrote: dict with lds_bytes, kind, build_flags, ... (the
+    fields of compile_matmul that belong to the file; kernel_name, grid and block are not among them)."""
+    info = KernelInfo()
+    check(lib().kcg_code_object_info(str(code_path).encode(), ctypes.byref(info)))
+    d = _info_dict(info)
+    for k in ("kernel_name", "grid", "block", "cache_hit"):
+        d.pop(k)
+    return d
+
+
+def compiler_identity():
+    """"hiprtc:<library path>:<size>" of the compiler the next compile uses ($KCG_HIPRTC_LIB selects another)."""
+    buf = ctypes.create_string_buffer(2048)
+    check(lib().kcg_compiler_identity(buf, len(buf)))
+    return buf.value.decode()
+
+
+class use_hiprtc:
+    """Context manager: compiles inside it use the hiprtc library at `path` (None: the process's own).  The
+    library reads $KCG_HIPRTC_LIB at every compile and keeps such a compiler in a link namespace of its own."""
+
+    def __init__(self, path):
+        self.path = path
+
+    def __enter__(self):
+        self.old = os.environ.get("KCG_HIPRTC_LIB")
+        if self.path:
+            os.environ["KCG_HIPRTC_LIB"] = self.path
+        else:
+            os.environ.pop("KCG_HIPRTC_LIB", None)
+        return self
+
+    def __exit__(self, *exc):
+        if self.old is None:
+            os.environ.pop("KCG_HIPRTC_LIB", None)
+        else:
+            os.environ["KCG_HIPRTC_LIB"] = self.old
+        return False
 
 
 def load(code_path, kernel_name_, lds_bytes, device):

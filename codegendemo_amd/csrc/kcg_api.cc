@@ -8,6 +8,9 @@
 //
 // There is no CPU execution path here: without a HIP device, load/launch/benchmark fail with
 // KCG_ERR_HIP.  Compilation alone needs no device.
+#ifndef _GNU_SOURCE
+#define _GNU_SOURCE   /* dlmopen */
+#endif
 #include <dlfcn.h>
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
@@ -18,9 +21,12 @@
 #include <algorithm>
 #include <atomic>
 #include <cerrno>
+#include <climits>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -28,7 +34,7 @@
 
 #include "kcg_config.h"
 
-#define KCG_VERSION "kcg-gemm-gfx950 0.2"
+#define KCG_VERSION "kcg-gemm-gfx950 0.3"
 
 // The device template headers, embedded at build time (directory given by -DKCG_DEVICE_HEADER_DIR):
 // kcg_gemm_device.h is what the instantiation stub includes; it includes the others.
@@ -62,14 +68,41 @@ thread_local std::string g_err;
 struct LoadedFunction {
   int n_args;
   uint64_t module;
+  int es_a, es_b, es_c;   // element sizes of A, B, C from the DTabc part of the kernel name; 0: not known
 };
 std::mutex g_loaded_mu;
 std::unordered_map<uint64_t, LoadedFunction> g_loaded;
 
-int loaded_args(uint64_t function) {
+LoadedFunction loaded_function(uint64_t function) {
   std::lock_guard<std::mutex> lock(g_loaded_mu);
   auto it = g_loaded.find(function);
-  return it == g_loaded.end() ? 0 : it->second.n_args;
+  return it == g_loaded.end() ? LoadedFunction{0, 0, 0, 0, 0} : it->second;
+}
+int loaded_args(uint64_t function) { return loaded_function(function).n_args; }
+
+// "..._DTabcfloat16xfloat16xfloat32_..." -> 2, 2, 4 (0 where the name does not say)
+void element_sizes_from_name(const std::string& name, int es[3]) {
+  es[0] = es[1] = es[2] = 0;
+  size_t p = name.find("DTabc");
+  if (p == std::string::npos) return;
+  p += 5;
+  for (int i = 0; i < 3; ++i) {
+    static const struct { const char* text; int size; } types[] = {
+        {"float16", 2}, {"bfloat16", 2}, {"float32", 4}, {"float64", 8}};
+    for (const auto& t : types) {
+      const size_t n = strlen(t.text);
+      if (name.compare(p, n, t.text) == 0) {
+        es[i] = t.size;
+        p += n;
+        break;
+      }
+    }
+    if (!es[i]) return;
+    if (i < 2) {
+      if (p >= name.size() || name[p] != 'x') return;
+      ++p;
+    }
+  }
 }
 
 int fail(int code, const std::string& msg) {
@@ -160,11 +193,49 @@ const HipApi& hip_api() {
   return api;
 }
 
-const RtcApi& rtc_api() {
-  static const RtcApi api = [] {
-    RtcApi a;
-    void* h = open_shared("libhiprtc.so.7", &a.error);
-    if (!h) return a;
+// Which hiprtc compiles.  Default: the one the process already carries, else the system's (open_shared).
+// $KCG_HIPRTC_LIB = path of another libhiprtc: that library is opened in a link namespace of its own
+// (dlmopen), so that the compiler library it loads by name (libamd_comgr.so.3) is the one that lies beside
+// it and not a copy of the same name the process has already loaded.  This is how one process (a Python
+// process with PyTorch's bundled ROCm, say) builds kernels with the system's compiler as well, e.g. to put
+// both builds through the same correctness gate.  Read at every compile.
+// `identity` goes into the cache key: hiprtcVersion() alone does not tell two ROCm releases apart.
+struct RtcLib {
+  RtcApi api;
+  std::string identity;
+};
+
+std::string library_identity(void* symbol) {
+  Dl_info info;
+  if (!symbol || !dladdr(symbol, &info) || !info.dli_fname) return "hiprtc:?";
+  char real[PATH_MAX];
+  std::string path = realpath(info.dli_fname, real) ? real : info.dli_fname;
+  struct stat st;
+  long size = stat(path.c_str(), &st) == 0 ? (long)st.st_size : -1;
+  return "hiprtc:" + path + ":" + std::to_string(size);
+}
+
+const RtcLib& rtc_lib() {
+  static std::mutex mu;
+  static std::map<std::string, std::unique_ptr<RtcLib>> libs;
+  const char* v = getenv("KCG_HIPRTC_LIB");
+  const std::string which = (v && *v) ? v : "";
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = libs.find(which);
+  if (it != libs.end()) return *it->second;
+  std::unique_ptr<RtcLib> lib(new RtcLib);
+  RtcApi& a = lib->api;
+  void* h = nullptr;
+  if (which.empty()) {
+    h = open_shared("libhiprtc.so.7", &a.error);
+  } else {
+    h = dlmopen(LM_ID_NEWLM, which.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!h) {
+      const char* why = dlerror();
+      a.error = " cannot load $KCG_HIPRTC_LIB=" + which + ": " + (why ? why : "?");
+    }
+  }
+  if (h) {
     bool all = true;
 #define X(name)                                                              \
   a.p_##name = reinterpret_cast<decltype(&::name)>(dlsym(h, KCG_STR(name))); \
@@ -172,13 +243,12 @@ const RtcApi& rtc_api() {
     KCG_RTC_FUNCS(X)
 #undef X
     a.ok = all;
-    return a;
-  }();
-  return api;
+    lib->identity = library_identity(reinterpret_cast<void*>(a.p_hiprtcVersion));
+  }
+  return *(libs[which] = std::move(lib));
 }
 
 #define HIPF(name) (hip_api().p_##name)
-#define RTCF(name) (rtc_api().p_##name)
 
 // Same text shape as the reference loader's errors (loaderCCode/hip.c:8-21).
 int hip_fail(hipError_t e, const char* what) {
@@ -424,12 +494,10 @@ int kcg_instantiation_source(const kcg_matmul_cfg* cfg, int kind, char* out, int
   return copy_out(kcg::instantiation_source(c, k, env_flag("KCG_XCD_REMAP", true)), out, out_len);
 }
 
-// Scratch (private segment) bytes per lane of the kernel in a code object, from its metadata note:
-// the msgpack key ".private_segment_fixed_size" is followed by its unsigned value.  -1 when the key is
-// not there (the caller then does not know).
-static long code_object_scratch_bytes(const std::vector<char>& code) {
-  static const char key[] = ".private_segment_fixed_size";
-  const size_t klen = sizeof(key) - 1;
+// What the metadata note of a code object says about its (one) kernel: the msgpack key is followed by its
+// unsigned value.  -1 where the key is not there (the caller then does not know).
+static long code_object_meta(const std::vector<char>& code, const char* key) {
+  const size_t klen = strlen(key);
   for (size_t i = 0; i + klen + 1 <= code.size(); ++i) {
     if (memcmp(code.data() + i, key, klen) != 0) continue;
     const unsigned char* p = reinterpret_cast<const unsigned char*>(code.data()) + i + klen;
@@ -447,8 +515,47 @@ static long code_object_scratch_bytes(const std::vector<char>& code) {
   return -1;
 }
 
+struct CodeMeta {
+  long scratch, vgprs, vgpr_spills, sgpr_spills;
+  static CodeMeta of(const std::vector<char>& code) {
+    return CodeMeta{code_object_meta(code, ".private_segment_fixed_size"), code_object_meta(code, ".vgpr_count"),
+                    code_object_meta(code, ".vgpr_spill_count"), code_object_meta(code, ".sgpr_spill_count")};
+  }
+  bool known() const { return scratch >= 0 && vgprs >= 0; }
+  // the register allocator ran out of vector registers: scratch memory in use, vector registers spilled, or the
+  // whole file of 512 taken.  (Scalar registers spilled into lanes of a vector register alone do not count: that
+  // is what the compiler does in every large kernel, 110 of 1900 cached instantiations, none of them ever wrong.)
+  bool under_pressure() const { return !known() || scratch != 0 || vgpr_spills > 0 || vgprs >= 512; }
+};
+
 // Outcome of build_variant besides the kcg_status values: the direct-staging build would spill.
 static const int kBuildSpills = 1;
+
+// -DKCG_DIAG_...: builds of the direct-staging kernel that leave work out on purpose (their C is wrong)
+static bool has_diagnostic_flag(const std::vector<std::string>& flags) {
+  for (const auto& f : flags)
+    if (f.find("KCG_DIAG_") != std::string::npos) return true;
+  return false;
+}
+
+// "<name>.<hash>.buildinfo" beside a cached code object: what kcg_kernel_info reports about the build
+static void write_build_info(const std::string& path, const kcg_kernel_info& k) {
+  char text[200];
+  const int n = snprintf(text, sizeof(text), "build_flags=%d scratch_bytes=%d vgprs=%d sgpr_spills=%d lds_bytes=%d kind=%d\n",
+                         k.build_flags, k.scratch_bytes, k.vgprs, k.sgpr_spills, k.lds_bytes, k.kind);
+  write_file_atomic(path, text, (size_t)n);
+}
+static bool read_build_info(const std::string& path, kcg_kernel_info* k) {
+  std::vector<char> raw;
+  if (!read_file(path, &raw)) return false;
+  raw.push_back(0);
+  int f = 0, sc = 0, vg = 0, sg = 0, lds = 0, kind = 0;
+  if (sscanf(raw.data(), "build_flags=%d scratch_bytes=%d vgprs=%d sgpr_spills=%d lds_bytes=%d kind=%d", &f, &sc, &vg, &sg, &lds,
+             &kind) != 6)
+    return false;
+  k->build_flags = f; k->scratch_bytes = sc; k->vgprs = vg; k->sgpr_spills = sg; k->lds_bytes = lds; k->kind = kind;
+  return true;
+}
 
 // Builds (or finds in the cache) the code object of config c as kernel family k; `allow_direct` lets a
 // matrix-core config that is eligible for direct global->LDS staging use that kernel.
@@ -456,8 +563,11 @@ static const int kBuildSpills = 1;
 static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, const std::string& arch, int ex, kcg_kernel_info* out) {
   const bool xcd = env_flag("KCG_XCD_REMAP", true);
   const bool direct = allow_direct && k == KCG_KIND_MFMA && kcg::mfma_direct(c);
+  const bool declined = !allow_direct && k == KCG_KIND_MFMA && kcg::mfma_direct(c);
   const std::string name = ex < 0 ? kcg::kernel_name(c) : kcg::kernel_name_ex(c, ex);
   const std::string stub = kcg::instantiation_source(c, k, xcd, allow_direct, ex);
+  const std::vector<std::string> extra = extra_flags();
+  const bool diagnostic = has_diagnostic_flag(extra);
 
   memset(out, 0, sizeof(*out));
   if (name.size() >= sizeof(out->kernel_name)) return fail(KCG_ERR_ARGUMENT, "kernel name too long");
@@ -468,16 +578,26 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
   out->block[1] = out->block[2] = 1;
   out->lds_bytes = kcg::lds_bytes(c, k, allow_direct);
   out->kind = k;
+  out->scratch_bytes = out->vgprs = out->sgpr_spills = -1;
 
-  if (!rtc_api().ok) return fail(KCG_ERR_COMPILE, "hiprtc unavailable:" + rtc_api().error);
+  // A build that computes a wrong C on purpose must be asked for twice: by its flag and by $KCG_ALLOW_DIAG=1
+  // (the reference's comparable hook, an LLVM pass plugin named in the environment, is opt-in as well:
+  // LLVMIRTranslation.cc:98-108).  Such a kernel keeps the reference name; kcg_kernel_info says what it is.
+  if (diagnostic && !env_flag("KCG_ALLOW_DIAG", false))
+    return fail(KCG_ERR_ARGUMENT, "$KCG_EXTRA_FLAGS asks for a diagnostic build (-DKCG_DIAG_...: the kernel leaves work out and its "
+                                  "result is wrong on purpose); set KCG_ALLOW_DIAG=1 to build it");
+
+  const RtcLib& rtc = rtc_lib();           // one compiler for the whole call, whatever happens to the environment
+  if (!rtc.api.ok) return fail(KCG_ERR_COMPILE, "hiprtc unavailable:" + rtc.api.error);
+#define RTC(name) (rtc.api.p_##name)
   std::string flags_text;
   for (const auto& f : compile_flags()) flags_text += f + " ";
   {
     int major = 0, minor = 0;
-    RTCF(hiprtcVersion)(&major, &minor);
-    flags_text += "hiprtc" + std::to_string(major) + "." + std::to_string(minor);
+    RTC(hiprtcVersion)(&major, &minor);
+    flags_text += "hiprtc" + std::to_string(major) + "." + std::to_string(minor) + " " + rtc.identity + " ";
   }
-  for (const auto& f : extra_flags()) flags_text += f + " ";
+  for (const auto& f : extra) flags_text += f + " ";
   if (!env_flag("KCG_SPILL_REBUILD", true)) flags_text += "first-build-kept ";
   uint64_t h = fnv1a(KCG_VERSION);
   h = fnv1a(arch, h);
@@ -489,14 +609,16 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
 
   const std::string dir = cache_dir();
   if (!make_dirs(dir)) return fail(KCG_ERR_IO, "cannot create cache directory " + dir);
-  const std::string path = dir + "/" + name + "." + hex + ".hsaco";
+  const std::string stem = dir + "/" + name + "." + hex;
+  const std::string path = stem + ".hsaco";
   if (path.size() >= sizeof(out->code_path)) return fail(KCG_ERR_IO, "code object path too long");
   memcpy(out->code_path, path.c_str(), path.size() + 1);
   // remembers that this very build (same sources, flags, compiler) spilled: no need to compile it again
-  const std::string spill_marker = dir + "/" + name + "." + hex + ".spills";
+  const std::string spill_marker = stem + ".spills";
+  const std::string info_path = stem + ".buildinfo";
 
   if (!env_flag("KCG_CACHE_BYPASS", false)) {
-    if (file_exists(path)) {
+    if (file_exists(path) && read_build_info(info_path, out)) {
       out->cache_hit = 1;
       g_err.clear();
       return KCG_OK;
@@ -507,89 +629,124 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
   // one hiprtc build of the stub with the engine's flags, $KCG_EXTRA_FLAGS and `more` behind them
   auto compile = [&](const std::vector<std::string>& more, std::vector<char>* code) -> int {
     hiprtcProgram prog;
-    hiprtcResult r = RTCF(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", kNumDeviceHeaders,
-                                               const_cast<const char**>(kDeviceHeaderSrcs),
-                                               const_cast<const char**>(kDeviceHeaderNames));
-    if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTCF(hiprtcGetErrorString)(r));
+    hiprtcResult r = RTC(hiprtcCreateProgram)(&prog, stub.c_str(), "kcg_instance.hip", kNumDeviceHeaders,
+                                              const_cast<const char**>(kDeviceHeaderSrcs),
+                                              const_cast<const char**>(kDeviceHeaderNames));
+    if (r != HIPRTC_SUCCESS) return fail(KCG_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + RTC(hiprtcGetErrorString)(r));
     std::vector<std::string> opts = compile_flags();
     opts.push_back("--offload-arch=" + arch);
-    for (const auto& f : extra_flags()) opts.push_back(f);
+    for (const auto& f : extra) opts.push_back(f);
     for (const auto& f : more) opts.push_back(f);
     std::vector<const char*> optv;
     for (const auto& o : opts) optv.push_back(o.c_str());
-    r = RTCF(hiprtcCompileProgram)(prog, (int)optv.size(), optv.data());
+    r = RTC(hiprtcCompileProgram)(prog, (int)optv.size(), optv.data());
     if (r != HIPRTC_SUCCESS) {
       size_t n = 0;
-      RTCF(hiprtcGetProgramLogSize)(prog, &n);
+      RTC(hiprtcGetProgramLogSize)(prog, &n);
       std::string log(n, 0);
-      if (n) RTCF(hiprtcGetProgramLog)(prog, &log[0]);
-      RTCF(hiprtcDestroyProgram)(&prog);
-      return fail(KCG_ERR_COMPILE, std::string("hiprtc: ") + RTCF(hiprtcGetErrorString)(r) + " for " + name + "\n" + log);
+      if (n) RTC(hiprtcGetProgramLog)(prog, &log[0]);
+      RTC(hiprtcDestroyProgram)(&prog);
+      return fail(KCG_ERR_COMPILE, std::string("hiprtc: ") + RTC(hiprtcGetErrorString)(r) + " for " + name + "\n" + log);
     }
     size_t n = 0;
-    r = RTCF(hiprtcGetCodeSize)(prog, &n);
+    r = RTC(hiprtcGetCodeSize)(prog, &n);
     code->assign(n, 0);
-    if (r == HIPRTC_SUCCESS) r = RTCF(hiprtcGetCode)(prog, code->data());
-    RTCF(hiprtcDestroyProgram)(&prog);
+    if (r == HIPRTC_SUCCESS) r = RTC(hiprtcGetCode)(prog, code->data());
+    RTC(hiprtcDestroyProgram)(&prog);
     if (r != HIPRTC_SUCCESS || n == 0) return fail(KCG_ERR_COMPILE, "hiprtc returned no code object");
     return KCG_OK;
   };
+#undef RTC
   std::vector<char> code;
   if (int rc = compile({}, &code)) return rc;
+  CodeMeta meta = CodeMeta::of(code);
+  std::string note;
   // The direct-staging kernel reads LDS with instructions the compiler does not know to be
   // asynchronous: a fragment register spilled to scratch memory would be stored before its data has
   // arrived.  Such a build is never used (nor cached): the caller falls back to register staging.
   // (a code object whose metadata does not say counts as spilling: the kernel is not used unverified)
-  if (direct && code_object_scratch_bytes(code) != 0) {
-    const char note[] = "direct-staging build needs scratch memory (register spills); register staging is used instead\n";
-    write_file_atomic(spill_marker, note, sizeof(note) - 1);
+  if (direct && (!meta.known() || meta.scratch != 0 || meta.vgpr_spills > 0)) {
+    const char text[] = "direct-staging build needs scratch memory (register spills); register staging is used instead\n";
+    write_file_atomic(spill_marker, text, sizeof(text) - 1);
     return kBuildSpills;
   }
-  // A register-staged or scalar kernel that does not fit the register file without spilling is built once
-  // more at -O1, and that build is the one kept.  One such kernel (fp64, one wave on a 64x64x64 tile with
-  // both prefetch flags, M=8 N=208 K=592: 512 registers and 1 KiB of scratch per lane) returns wrong sums at
-  // -O2 and -O3 and the right ones at -O1, as do all spilling kernels of a 1000-config random sample (184 of
-  // them, 9 % slower at the median).  Such configs never win a tuning run; they must still be right.
-  // $KCG_SPILL_REBUILD=0 keeps the first build.
-  if (!direct && code_object_scratch_bytes(code) != 0 && env_flag("KCG_SPILL_REBUILD", true)) {
+  // OPEN DEFECT, worked around: a register-staged or scalar kernel that the register allocator could not fit
+  // (CodeMeta::under_pressure) is built once more at -O1, and that build is the one kept.  One such kernel
+  // (fp64, one wave on a 64x64x64 tile with both prefetch flags, M=8 N=208 K=592: 512 registers, 1 KiB of
+  // scratch per lane) returns wrong sums at -O2 and -O3 and the right ones at -O1; the cause inside the compiler
+  // is not known.  All spilling kernels of a 1000-config random sample (184 of them) are right at -O1 and run
+  // 9 % slower at the median.  Such configs never win a tuning run; they must still be right.
+  // kcg_kernel_info.build_flags says which build a caller got.  $KCG_SPILL_REBUILD=0 keeps the first build.
+  if (!direct && meta.under_pressure() && env_flag("KCG_SPILL_REBUILD", true)) {
     std::vector<char> calm;
     if (int rc = compile({"-O1"}, &calm)) return rc;
     code.swap(calm);
+    out->build_flags |= KCG_BUILD_LOW_OPT;
+    if (!meta.known()) {
+      out->build_flags |= KCG_BUILD_META_UNKNOWN;
+      note = "note: the code object's metadata does not state its register use; the kernel was rebuilt at -O1 as if it spilled";
+    }
+    meta = CodeMeta::of(code);
   }
+  if (diagnostic) {
+    out->build_flags |= KCG_BUILD_DIAGNOSTIC;
+    note = "note: diagnostic build (" + std::string(getenv("KCG_EXTRA_FLAGS")) + "): the result of this kernel is wrong on purpose";
+  }
+  if (declined) out->build_flags |= KCG_BUILD_DIRECT_DECLINED;
+  out->scratch_bytes = (int32_t)meta.scratch;
+  out->vgprs = (int32_t)meta.vgprs;
+  out->sgpr_spills = (int32_t)meta.sgpr_spills;
   if (!write_file_atomic(path, code.data(), code.size())) return fail(KCG_ERR_IO, "cannot write " + path);
+  write_build_info(info_path, *out);
   if (env_flag("KCG_KEEP_SOURCE", false)) {
-    std::string sp = dir + "/" + name + "." + hex + ".hip";
+    std::string sp = stem + ".hip";
     write_file_atomic(sp, stub.data(), stub.size());
   }
+  g_err = note;
+  return KCG_OK;
+}
+
+static int compile_entry(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, int ex, kcg_kernel_info* out) {
+  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
+  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
+  std::string why;
+  int k = resolve_kind(c, kind, &why);
+  if (k < 0) return fail(k, "invalid config: " + why);
+  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
+  int r = build_variant(c, k, /*allow_direct=*/true, arch, ex, out);
+  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, ex, out);
+  return r;
+}
+
+int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, kcg_kernel_info* out) {
+  return compile_entry(cfg, arch_in, kind, -1, out);
+}
+
+int kcg_compile_matmul_ex(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, int epilogue, kcg_kernel_info* out) {
+  if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_ALPHA_BETA) return fail(KCG_ERR_ARGUMENT, "unknown epilogue");
+  return compile_entry(cfg, arch_in, kind, epilogue, out);
+}
+
+int kcg_code_object_info(const char* code_path, kcg_kernel_info* out) {
+  if (!code_path || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
+  std::string p = code_path;
+  const std::string ext = ".hsaco";
+  if (p.size() <= ext.size() || p.compare(p.size() - ext.size(), ext.size(), ext) != 0)
+    return fail(KCG_ERR_ARGUMENT, "not a code object of this library (no .hsaco suffix): " + p);
+  memset(out, 0, sizeof(*out));
+  if (p.size() >= sizeof(out->code_path)) return fail(KCG_ERR_IO, "code object path too long");
+  memcpy(out->code_path, p.c_str(), p.size() + 1);
+  if (!read_build_info(p.substr(0, p.size() - ext.size()) + ".buildinfo", out))
+    return fail(KCG_ERR_IO, "no build record beside " + p + " (the code object was not written by kcg_compile_matmul)");
   g_err.clear();
   return KCG_OK;
 }
 
-int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, kcg_kernel_info* out) {
-  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
-  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
-  std::string why;
-  int k = resolve_kind(c, kind, &why);
-  if (k < 0) return fail(k, "invalid config: " + why);
-  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
-  int r = build_variant(c, k, /*allow_direct=*/true, arch, -1, out);
-  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, -1, out);
-  return r;
+int kcg_compiler_identity(char* out, int out_len) {
+  const RtcLib& rtc = rtc_lib();
+  if (!rtc.api.ok) return fail(KCG_ERR_COMPILE, "hiprtc unavailable:" + rtc.api.error);
+  return copy_out(rtc.identity, out, out_len);
 }
-
-int kcg_compile_matmul_ex(const kcg_matmul_cfg* cfg, const char* arch_in, int kind, int epilogue, kcg_kernel_info* out) {
-  if (!cfg || !out) return fail(KCG_ERR_ARGUMENT, "null argument");
-  if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_ALPHA_BETA) return fail(KCG_ERR_ARGUMENT, "unknown epilogue");
-  kcg::MatmulConfig c = kcg::MatmulConfig::from(*cfg);
-  std::string why;
-  int k = resolve_kind(c, kind, &why);
-  if (k < 0) return fail(k, "invalid config: " + why);
-  const std::string arch = (arch_in && *arch_in) ? arch_in : "gfx950";
-  int r = build_variant(c, k, /*allow_direct=*/true, arch, epilogue, out);
-  if (r == kBuildSpills) r = build_variant(c, k, /*allow_direct=*/false, arch, epilogue, out);
-  return r;
-}
-
 
 int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int device, uint64_t* module,
              uint64_t* function, int32_t* n_regs, int32_t* n_spills) {
@@ -628,8 +785,10 @@ int kcg_load(const char* code_path, const char* kernel_name, int lds_bytes, int 
       const size_t n = strlen(suffix);
       return name.size() >= n && name.compare(name.size() - n, n, suffix) == 0;
     };
+    int es[3];
+    element_sizes_from_name(name, es);
     std::lock_guard<std::mutex> lock(g_loaded_mu);
-    g_loaded[*function] = LoadedFunction{(ends("EX_") || ends("EXab_")) ? 8 : 3, *module};
+    g_loaded[*function] = LoadedFunction{(ends("EX_") || ends("EXab_")) ? 8 : 3, *module, es[0], es[1], es[2]};
   }
   g_err.clear();
   return KCG_OK;
@@ -663,7 +822,13 @@ int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t b
   if (grid[1] != 1 || grid[2] != 1) return fail(KCG_ERR_ARGUMENT, "the batch goes on grid[1]: grid must be {n, 1, 1}");
   if (!a || !b || !c) return fail(KCG_ERR_ARGUMENT, "null device pointer");
   if ((a | b | c) & 15) return fail(KCG_ERR_ARGUMENT, "a, b and c must be 16-byte aligned");
-  if (loaded_args(function) == 3) return fail(KCG_ERR_ARGUMENT, "this kernel has the three-pointer form: use kcg_launch");
+  const LoadedFunction lf = loaded_function(function);
+  if (lf.n_args == 3) return fail(KCG_ERR_ARGUMENT, "this kernel has the three-pointer form: use kcg_launch");
+  // problem z starts stride * z elements into each buffer and must be as aligned as problem 0: the kernels move
+  // 16-byte vectors relative to the start of a matrix
+  if (batch > 1 && ((stride_a * lf.es_a) % 16 || (stride_b * lf.es_b) % 16 || (stride_c * lf.es_c) % 16))
+    return fail(KCG_ERR_ARGUMENT, "stride_a, stride_b and stride_c must be multiples of 16 bytes (every problem of a batch "
+                                  "must start 16-byte aligned)");
   void* pa = (void*)(uintptr_t)a;
   void* pb = (void*)(uintptr_t)b;
   void* pc = (void*)(uintptr_t)c;

@@ -108,6 +108,10 @@ std::string check_common(const MatmulConfig& c) {
   if (!is_pow2(c.GLW_A) || !is_pow2(c.GLW_B)) return "GLOB_LOAD_WIDTH_A/B must be a power of two >= 1";
   if (c.GLW_A * sz > 16 || c.GLW_B * sz > 16) return "GLOB_LOAD_WIDTH_A/B wider than 128 bits";
   if (!is_pow2(c.GSW) || c.GSW * dtype_size(c.dtC) > 16) return "GLOB_STORE_WIDTH must be a power of two, at most 128 bits";
+  // a lane whose vector lies outside the matrix reads the first vector of the buffer instead and drops it: every
+  // operand must hold at least one 16-byte vector
+  if ((long)c.M * c.K * sz < 16 || (long)c.K * c.N * sz < 16 || (long)c.M * c.N * dtype_size(c.dtC) < 16)
+    return "A, B and C must each hold at least 16 bytes";
   return "";
 }
 

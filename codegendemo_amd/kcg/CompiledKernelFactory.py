@@ -17,13 +17,30 @@ class EnumOperator(Enum):
 
 class UserInputs:
     def __init__(self, hsaco_path: str, kernel_func_name: str, kernelParam: KernelArgMatmul):
+        """The reference builds this from (path, name, config) alone (KCGTask.py:293-296) and recomputes the LDS
+        size from the config (CompiledKernelFactory.py:30-44).  That formula does not describe this engine's
+        kernels (padded rows in the scalar kernel, fp32 partial sums for 16-bit split-U, static LDS in the
+        direct-staging kernel), so the size is taken from what the compile recorded beside the code object:
+        a file read, no compile, nothing from the environment.  A path that is not a code object of the engine
+        leaves m_ldsBytes unset, and sharedMem() then says so instead of guessing."""
         self.operatorKind = EnumOperator.Matmul
         self.hsacoPath = hsaco_path
         self.kernelFuncName = kernel_func_name
         self.kernelParam = kernelParam
         self.m_gridDims = [1, 1, 1]
         self.m_blockDims = [1, 1, 1]
-        self.m_ldsBytes = None      # set from the compile result when known
+        self.m_ldsBytes = None      # dynamic LDS of the launch
+        self.m_buildFlags = 0       # kcg_build_flag bits of the code object (_native.BUILD_*)
+        self.m_scratchBytes = -1    # scratch memory per lane (register spills); -1: unknown
+        from .. import _native
+        try:
+            rec = _native.code_object_info(hsaco_path)
+        except _native.KcgError:
+            rec = None
+        if rec is not None:
+            self.m_ldsBytes = rec["lds_bytes"]
+            self.m_buildFlags = rec["build_flags"]
+            self.m_scratchBytes = rec["scratch_bytes"]
 
     def gridDims(self):
         return self.m_gridDims
@@ -32,22 +49,10 @@ class UserInputs:
         return self.m_blockDims
 
     def sharedMem(self):
-        """Dynamic LDS bytes for the launch: what the kernel inside the code object needs, as the engine
-        reported it at compile time (m_ldsBytes).  A driver written for the reference builds UserInputs from
-        (path, name, config) alone (KCGTask.py:293-296) and relies on the reference's formula
-        (CompiledKernelFactory.py:30-44) here; that formula does not describe this engine's kernels (padded
-        rows in the scalar kernel, fp32 partial sums for 16-bit split-U, static LDS in the direct-staging
-        kernel), so the engine is asked instead: the compile is a cache hit that returns the figure that
-        belongs to exactly this code object.  A code object the engine would not produce for this config
-        (another kernel family was forced) is refused rather than launched with a guessed size."""
-        if self.m_ldsBytes is not None:
-            return int(self.m_ldsBytes)
-        from .. import _native
-        info = _native.compile_matmul(self.kernelParam.values())
-        if info["code_path"] != self.hsacoPath or info["kernel_name"] != self.kernelFuncName:
-            raise ValueError("UserInputs.sharedMem(): the LDS size of this code object is unknown (it is not what "
-                             "the engine builds for this config by default); set m_ldsBytes from the compile result")
-        self.m_ldsBytes = info["lds_bytes"]
+        """Dynamic LDS bytes for the launch (no side effects)."""
+        if self.m_ldsBytes is None:
+            raise ValueError(f"UserInputs.sharedMem(): {self.hsacoPath} has no build record beside it (it was not written "
+                             "by this engine's compile); set m_ldsBytes to the kernel's dynamic LDS size")
         return int(self.m_ldsBytes)
 
     def numCTA(self):

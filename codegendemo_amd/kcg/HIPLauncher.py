@@ -44,6 +44,14 @@ class HIPLauncher:
                 if hasattr(x, "is_contiguous") and not x.is_contiguous():
                     raise ValueError(f"operand {label} must be contiguous")
 
+    @staticmethod
+    def _check_strides(args, batch, strides):
+        """Every problem's buffers must be as aligned as the first one's: the kernels move 16-byte vectors
+        (kcg_launch_batched refuses such strides too; here the message names the operand)."""
+        for label, x, stride in zip("abc", args, strides):
+            if batch > 1 and hasattr(x, "element_size") and (int(stride) * int(x.element_size())) % 16:
+                raise ValueError(f"stride_{label} = {stride} elements is not a multiple of 16 bytes")
+
     def launchKernel(self, devId: int, *args):
         if self.m_kernelLib.m_kernelFuncName.endswith(("EX_", "EXab_")):
             raise TypeError("a kernel in the batched-strided form takes strides, alpha and beta: use run_batched")
@@ -58,10 +66,7 @@ class HIPLauncher:
             raise TypeError("this kernel was not compiled in the batched-strided form (KCGCompiler(epilogue=...))")
         if batch > 0:
             self._check_operands((a, b, c), batch, (stride_a, stride_b, stride_c))
-            # every problem's buffers must be as aligned as the first one's: the kernels move 16-byte vectors
-            for label, x, stride in zip("abc", (a, b, c), (stride_a, stride_b, stride_c)):
-                if batch > 1 and hasattr(x, "element_size") and (int(stride) * int(x.element_size())) % 16:
-                    raise ValueError(f"stride_{label} = {stride} elements is not a multiple of 16 bytes")
+            self._check_strides((a, b, c), batch, (stride_a, stride_b, stride_c))
         fn = self._function()
         a, b, c = (_device_address(x) for x in (a, b, c))
         _native.launch_batched(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,
@@ -81,6 +86,7 @@ class HIPLauncher:
         if not self.m_kernelLib.m_kernelFuncName.endswith(("EX_", "EXab_")):
             raise TypeError("this kernel was not compiled in the batched-strided form (KCGCompiler(epilogue=...))")
         self._check_operands((a, b, c), batch, (stride_a, stride_b, stride_c))
+        self._check_strides((a, b, c), batch, (stride_a, stride_b, stride_c))
         fn = self._function()
         a, b, c = (_device_address(x) for x in (a, b, c))
         return _native.benchmark_batched(fn, self.m_kernelLib.m_gridDims, self.m_kernelLib.m_blockDims, self.m_kernelLib.m_shmSize,

@@ -44,14 +44,18 @@ class KernelTestResult:
         self.diffRate = 0.0
         self.maxError = 0.0
         self.tflops = 0.0
+        self.nSpills = 0          # scratch dwords per lane of the kernel that was timed (0: no register spills)
+        self.lowOpt = False       # the kernel is the engine's -O1 rebuild of a build that ran out of registers
 
     def __str__(self):
         return "{" + f"correct : {self.isCorrect}, acc : {self.acc}, torchMs : {self.torch_elapseTimeMs}], config : {self.kpm}" + "}"
 
     def jsonfy(self) -> dict:
-        # schema of the reference's result log (KCGTask.py:39-46) + the absolute throughput
+        # schema of the reference's result log (KCGTask.py:39-46) + the absolute throughput and which build the
+        # timing belongs to (a kernel that spills registers, or the slower -O1 rebuild of one)
         return {"correct": bool(self.isCorrect), "acc": float(self.acc), "torchMs": float(self.torch_elapseTimeMs),
-                "kcgMs": float(self.kcg_elapseTimeMs), "tflops": float(self.tflops), "config": self.kpm.jsonfy()}
+                "kcgMs": float(self.kcg_elapseTimeMs), "tflops": float(self.tflops), "nSpills": int(self.nSpills),
+                "lowOpt": bool(self.lowOpt), "config": self.kpm.jsonfy()}
 
     def parseFromJson(self, jsonObj):
         self.isCorrect = jsonObj["correct"]
@@ -59,6 +63,8 @@ class KernelTestResult:
         self.torch_elapseTimeMs = jsonObj["torchMs"]
         self.kcg_elapseTimeMs = jsonObj["kcgMs"]
         self.tflops = jsonObj.get("tflops", 0.0)
+        self.nSpills = jsonObj.get("nSpills", 0)
+        self.lowOpt = jsonObj.get("lowOpt", False)
         self.kpm = KernelArgMatmul(0, 0, 0, 1, 1, 1)
         self.kpm.assignWithJson(jsonObj["config"])
 
@@ -195,6 +201,8 @@ class PerfTester:
                    nTorchEpsInitTest=50) -> KernelTestResult:
         import torch
         result = KernelTestResult(kpm)
+        result.lowOpt = bool(getattr(inConfig, "m_buildFlags", 0) & 1)       # _native.BUILD_LOW_OPT
+        result.nSpills = int(packedKernel.n_spills)
         dev = f"cuda:{PerfTester.currentDevId}"
         tc = inConfig.kernelParam.dtypeTorch('C')
         a, b = PerfTester._a, PerfTester._b

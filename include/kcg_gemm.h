@@ -77,7 +77,23 @@ typedef struct kcg_kernel_info {
   int32_t lds_bytes;     /* dynamic LDS to pass at launch                                          */
   int32_t kind;          /* kcg_kernel_kind actually chosen                                        */
   int32_t cache_hit;     /* 1 if the code object came from the on-disk cache                       */
+  int32_t build_flags;   /* kcg_build_flag bits: how this code object was built                    */
+  int32_t scratch_bytes; /* scratch memory per lane (register spills), -1: the code object does not say */
+  int32_t vgprs;         /* vector + accumulation registers per lane (of 512), -1: unknown          */
+  int32_t sgpr_spills;   /* scalar registers spilled into vector-register lanes, -1: unknown        */
 } kcg_kernel_info;
+
+/* How a code object was built (kcg_kernel_info.build_flags). */
+enum kcg_build_flag {
+  KCG_BUILD_LOW_OPT = 1,         /* built at -O1: the -O3 build ran out of vector registers (scratch memory, vector
+                                  * spills or all 512 registers taken); one such -O3 build is known to compute wrong
+                                  * sums, cause unknown, so none is handed out.  Typically ~10 % slower.           */
+  KCG_BUILD_DIAGNOSTIC = 2,      /* $KCG_EXTRA_FLAGS held a -DKCG_DIAG_ flag (needs KCG_ALLOW_DIAG=1): this kernel
+                                  * leaves work out and its result is WRONG on purpose                            */
+  KCG_BUILD_DIRECT_DECLINED = 4, /* the config selects the direct-staging kernel, but that build would spill: this is
+                                  * the register-staged kernel                                                    */
+  KCG_BUILD_META_UNKNOWN = 8     /* the code object's metadata did not state its register use (treated as spilling) */
+};
 
 /* ---- config semantics (host only, no GPU needed) ------------------------------------------- */
 
@@ -128,9 +144,25 @@ int kcg_block_mapping(const kcg_matmul_cfg* cfg, int bid, int xcd_remap, int32_t
  * KCG_ERR_INVALID_CONFIG: the config breaks a rule (text says which), nothing was compiled.
  * KCG_ERR_COMPILE: hiprtc failed.
  * A config that selects the direct-staging kernel but whose build would spill registers to scratch memory
- * (that kernel cannot tolerate spills) silently gets the register-staged kernel instead; a
- * "<name>.<hash>.spills" marker in the cache directory remembers the decision. */
+ * (that kernel cannot tolerate spills) gets the register-staged kernel instead (out->build_flags says so); a
+ * "<name>.<hash>.spills" marker in the cache directory remembers the decision.
+ * KCG_ERR_ARGUMENT: $KCG_EXTRA_FLAGS names a -DKCG_DIAG_ switch (a build that is wrong on purpose) without
+ * KCG_ALLOW_DIAG=1.  On KCG_OK kcg_last_error() is "" or a line that starts with "note:". */
 int kcg_compile_matmul(const kcg_matmul_cfg* cfg, const char* arch, int kind, kcg_kernel_info* out);
+
+/* What kcg_compile_matmul recorded about a code object it wrote (the "<name>.<hash>.buildinfo" file beside it):
+ * fills lds_bytes, kind, build_flags, scratch_bytes, vgprs and sgpr_spills of *out (code_path is copied, the other
+ * fields are zero).  Lets a caller that holds only (path, kernel name, config) — the reference's UserInputs,
+ * Runtime/python/kcg/CompiledKernelFactory.py:19-28, which recomputes the LDS size from the config — launch the
+ * kernel with the size that belongs to this very code object.  KCG_ERR_IO when there is no such record. */
+int kcg_code_object_info(const char* code_path, kcg_kernel_info* out);
+
+/* Which compiler kcg_compile_matmul uses right now: "hiprtc:<path of the library>:<its size>" (part of the cache
+ * key: hiprtcVersion() does not tell ROCm releases apart).  Default: the hiprtc the process already carries, else
+ * the system's.  $KCG_HIPRTC_LIB=<path of a libhiprtc.so> selects another one, loaded in a link namespace of
+ * its own so that it brings its own compiler library along; read at every compile.  The reference's counterpart
+ * is the fixed LLVM it links (src/lib/Target/HSACOTranslation.cc:153-257).  Returns the length or a negative status. */
+int kcg_compiler_identity(char* out, int out_len);
 
 /* ---- batched / strided GEMM with an alpha-beta epilogue ---------------------------------------------
  * The reference has neither: it lists batched GEMM as the next step of its roadmap (结果汇总.md:21-22) and
@@ -150,6 +182,8 @@ int kcg_compile_matmul_ex(const kcg_matmul_cfg* cfg, const char* arch, int kind,
 /* Launches `batch` problems of a kernel built by kcg_compile_matmul_ex: grid = {info.grid[0], batch, 1}.
  * stride_* are in elements of the respective buffer; stride_a or stride_b may be 0 (one operand shared by
  * the whole batch), stride_c may not (unless batch == 1).  batch <= 65535; batch == 0 launches nothing.
+ * For batch > 1 every stride must be a multiple of 16 bytes (stride * element size): each problem has to start as
+ * aligned as the first one (checked for functions that kcg_load handed out; KCG_ERR_ARGUMENT otherwise).
  * alpha and beta are read only by a kernel with KCG_EPILOGUE_ALPHA_BETA.  Asynchronous on `stream`. */
 int kcg_launch_batched(uint64_t function, const int32_t grid[3], const int32_t block[3], int lds_bytes,
                        uint64_t stream, uint64_t a, uint64_t b, uint64_t c, int32_t batch,

@@ -158,6 +158,9 @@ def test_invalid_configs_are_reported_not_compiled():
         "2^30": dict(good, M_SIZE=2**31 - 1),                               # rows are indexed with 32-bit integers
         "blocks": dict(good, M_SIZE=2**30, N_SIZE=2**30),
         "1024": dict(make_config(1024, 1024, 1024, BM=256, BN=256, BK=16, TM=8, TN=8), LOCAL_SPLIT_U=2),
+        # an operand smaller than one 16-byte vector: a lane outside the matrix reads the first vector of the buffer
+        "at least 16 bytes": dict(good, M_SIZE=1, N_SIZE=3, K_SIZE=64),     # C: 3 floats
+        "16 bytes": dict(good, M_SIZE=1, N_SIZE=64, K_SIZE=3),              # A: 3 floats
     }
     for needle, cfg in cases.items():
         v = vals(cfg)

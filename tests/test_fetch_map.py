@@ -1,7 +1,7 @@
 """The fetch map of the direct-staging kernel, walked on the host with the kernel's own code.
 
 FetchMap (kcg_device_direct.h) says which 16 bytes of A and B every lane's fetch instructions bring to LDS; it is
-written as host-callable code, so csrc/kcg_fetch_check.h, appended to the `struct Cfg` of an instantiation stub and
+written as host-callable code, so tests/kcg_fetch_check.h, appended to the `struct Cfg` of an instantiation stub and
 compiled for the host, can walk every block, K tile, wave, instruction and lane of a problem and check that no
 fetch leaves the operand buffers (the extents below put the ends of rows and of the buffers at every position
 inside a 16-byte chunk, with rows that start 2, 4, ... bytes off a 16-byte boundary) and that every element that
@@ -16,7 +16,8 @@ from codegendemo_amd import _native
 from codegendemo_amd.kcg.ConfigGenerator import make_config
 from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
 
-CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "codegendemo_amd", "csrc")
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(HERE), "codegendemo_amd", "csrc")
 HIPCC = "/opt/rocm/bin/hipcc"
 DIRECT = dict(shared_prefetch=1, reg_prefetch=1)
 # (dtype, tile kwargs)
@@ -56,7 +57,7 @@ def run_check(job):
     path = os.path.join(workdir, f"check_{index}")
     with open(path + ".hip", "w") as f:
         f.write(src)
-    p = subprocess.run([HIPCC, "--cuda-host-only", "-O1", "-std=c++17", "-include", "hip/hip_runtime.h", "-I", CSRC,
+    p = subprocess.run([HIPCC, "--cuda-host-only", "-O1", "-std=c++17", "-include", "hip/hip_runtime.h", "-I", CSRC, "-I", HERE,
                         "-o", path, path + ".hip"], capture_output=True, text=True)
     if p.returncode:
         return index, "compile failed: " + p.stderr[-1500:]

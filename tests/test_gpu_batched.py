@@ -204,6 +204,20 @@ def test_batched_benchmark_times_the_whole_batch(oracle):
     got = c_dev.cpu().numpy().reshape(batch, M, N)
     for z in range(batch):
         assert np.array_equal(got[z], 2.0 * oracle.matmul(a[z], b[z], a_trans=False))
+    # every problem of a batch must start 16-byte aligned: strides that are not are refused, by the Python launcher
+    # (which names the operand) and by the C entry points themselves, before anything is launched
+    with pytest.raises(ValueError, match="stride_a"):
+        kernel.benchmark_batched(a_dev, b_dev, c_dev, batch, M * K - 1, K * N, M * N)
+    with pytest.raises(ValueError, match="stride_c"):
+        kernel.run_batched(a_dev, b_dev, c_dev, batch, M * K, K * N, M * N - 2)
+    fn = kernel._info().m_function
+    for strides in ((M * K - 1, K * N, M * N), (M * K, K * N - 2, M * N), (M * K, K * N, M * N - 3)):
+        with pytest.raises(_native.KcgError, match="multiples of 16 bytes"):
+            _native.launch_batched(fn, kernel.gridDims, kernel.blockDims, kernel.shmSize, 0, a_dev.data_ptr(), b_dev.data_ptr(),
+                                   c_dev.data_ptr(), batch, *strides)
+    _native.launch_batched(fn, kernel.gridDims, kernel.blockDims, kernel.shmSize, 0, a_dev.data_ptr(), b_dev.data_ptr(),
+                           c_dev.data_ptr(), 1, M * K - 1, K * N - 1, M * N - 1)      # one problem: the strides are not used
+    torch.cuda.synchronize()
     kernel.unload()
     plain = build(make_config(M=128, N=192, K=64), SIMT, None)[1]          # a three-pointer kernel
     with pytest.raises(TypeError):

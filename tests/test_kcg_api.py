@@ -81,21 +81,32 @@ def test_compiler_return_shape_and_factory(tmp_path, monkeypatch):
     assert (gx, gy, gz, bx, by, bz) == (256, 1, 1, 256, 1, 1)
     assert KCGCompiler().compile_kernel_matmul(*kpm.values()) == res
     ui = UserInputs(path, name, kpm)
-    # a reference-style driver never sets m_ldsBytes (KCGTask.py:293-296): the engine is asked, not the formula
-    assert ui.m_ldsBytes is None
+    # a reference-style driver never sets m_ldsBytes (KCGTask.py:293-296): it comes from the record the compile
+    # left beside the code object, not from the reference's formula, and reading it compiles nothing
     comp = KCGCompiler()
     comp.compileKernel(kpm)
-    assert ui.sharedMem() == comp.lastInfo["lds_bytes"] == 2 * (64 + 64) * 16 * 4
-    # where formula and kernel disagree (row padding of the scalar kernel for A[M,K]) the engine's figure wins
+    assert ui.m_ldsBytes == ui.sharedMem() == comp.lastInfo["lds_bytes"] == 2 * (64 + 64) * 16 * 4
+    assert ui.m_buildFlags == 0 and ui.m_scratchBytes == 0
+    # where formula and kernel disagree (row padding of the scalar kernel for A[M,K]) the engine's figure wins, also
+    # for a kernel family that was forced: the record belongs to the file, not to the config
     kpm0 = kernelArgFromConfig(make_config(1024, 1024, 1024, shared_prefetch=1, is_atrans=0))
     comp.kind = 1
     p0, n0 = comp.compileKernel(kpm0)[0][:2]
-    forced = UserInputs(p0, n0, kpm0)
-    with pytest.raises(ValueError):
-        forced.sharedMem()              # not the default family for this config: unknown, refused
+    forced_lds = comp.lastInfo["lds_bytes"]
     comp.kind = 0
     p1, n1 = comp.compileKernel(kpm0)[0][:2]
+    assert p0 != p1 and forced_lds != comp.lastInfo["lds_bytes"]
+    assert UserInputs(p0, n0, kpm0).sharedMem() == forced_lds
     assert UserInputs(p1, n1, kpm0).sharedMem() == comp.lastInfo["lds_bytes"]
+    # a code object the engine did not write: the size is unknown and sharedMem() says so (no guess, no compile)
+    alien = tmp_path / "alien.hsaco"
+    alien.write_bytes(b"x")
+    stranger = UserInputs(str(alien), n0, kpm0)
+    assert stranger.m_ldsBytes is None
+    with pytest.raises(ValueError):
+        stranger.sharedMem()
+    stranger.m_ldsBytes = 4096
+    assert stranger.sharedMem() == 4096
     ui.m_gridDims, ui.m_blockDims = [gx, gy, gz], [bx, by, bz]
     assert ui.numCTA() == 256 and ui.operatorKind == EnumOperator.Matmul
     kernel = CompiledKernelFactory.getKernel(ui, 0)
