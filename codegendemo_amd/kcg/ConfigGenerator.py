@@ -62,6 +62,33 @@ def get_cfgs(tuning_cfg_file: str, engine_check: bool = True) -> list:
     return list(iter_cfgs(read_params(tuning_cfg_file), engine_check))
 
 
+def sample_cfgs(param_options: dict, n: int, seed: int, max_draws: int = 2000000):
+    """A seeded sample of what get_cfgs returns for a tuning space too large to enumerate (the reference's
+    GEMM_configs_1024.json spans some 10^8 raw points): points are drawn uniformly from the cartesian product
+    and pass through the same predicates as iter_cfgs.  Returns (valid, rejected): `valid` holds n points that
+    pass everything (each of them compiles); `rejected` the first n raw points that did not (the reference's
+    checker or the engine's predicate said no: the engine answers those with KCG_ERR_INVALID_CONFIG)."""
+    import random
+    rng = random.Random(seed)
+    keys = list(param_options.keys())
+    values = [v if isinstance(v, (list, tuple)) else [v] for v in param_options.values()]
+    chk = TuningSpaceChecker_Matmul
+    valid, rejected, seen = [], [], set()
+    for _ in range(max_draws):
+        if len(valid) >= n:
+            break
+        combo = tuple(rng.choice(v) for v in values)
+        if combo in seen:
+            continue
+        seen.add(combo)
+        cfg = _expand_dtype(dict(zip(keys, combo)))
+        if chk.check_warp(cfg) and chk.check_size(cfg) and chk.check_shm_size(cfg) and chk.check_engine(cfg):
+            valid.append(cfg)
+        elif len(rejected) < n:
+            rejected.append(cfg)
+    return valid, rejected
+
+
 def split_bigjson_to_temp(bigcfgs: dict, startIndex: int, endIndex: int, outDir: str) -> str:
     outDir = outDir.rstrip("/")
     part = {"cfgs": bigcfgs["cfgs"][startIndex:endIndex]}

@@ -11,10 +11,24 @@ from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
 NP_OF = {2: np.float16, 4: np.float32, 8: np.float64}
 
 
-def build_kernel(config, kind=_native.KIND_AUTO, device=0):
+def hiprtc_params():
+    """The compilers the bit-exact gates run under: the hiprtc the process carries (in a Python process the ROCm
+    that PyTorch bundles) and the system's (/opt/rocm: what a C program that links the library gets).  The
+    direct-staging kernel counts its LDS reads by hand and hides its matrix instructions from the compiler, so its
+    correctness has to be re-established per compiler; the two builds are separate cache entries."""
+    import os
+    import pytest
+    return [pytest.param(None, id="process-hiprtc"),
+            pytest.param(_native.SYSTEM_HIPRTC, id="system-hiprtc",
+                         marks=pytest.mark.skipif(not os.path.exists(_native.SYSTEM_HIPRTC), reason="no system ROCm"))]
+
+
+def build_kernel(config, kind=_native.KIND_AUTO, device=0, hiprtc=None):
+    """hiprtc: path of the hiprtc library that compiles (None: the process's own)."""
     kpm = kernelArgFromConfig(config)
     comp = KCGCompiler(kind=kind)
-    path, name, gx, gy, gz, bx, by, bz = comp.compileKernel(kpm)[0]
+    with _native.use_hiprtc(hiprtc):
+        path, name, gx, gy, gz, bx, by, bz = comp.compileKernel(kpm)[0]
     ui = UserInputs(path, name, kpm)
     ui.m_gridDims = [gx, gy, gz]
     ui.m_blockDims = [bx, by, bz]
@@ -28,11 +42,11 @@ def to_device(x, torch_dtype, device="cuda:0"):
     return torch.from_numpy(np.ascontiguousarray(x)).to(device=device, dtype=torch_dtype)
 
 
-def run_gemm(config, a_mk, b_kn, kind=_native.KIND_AUTO, poison=True):
+def run_gemm(config, a_mk, b_kn, kind=_native.KIND_AUTO, poison=True, hiprtc=None):
     """a_mk: logical [M,K] fp32 numpy, b_kn: [K,N].  Returns (C as float64-free numpy in the config's
     C dtype upcast to fp32, info).  The output buffer is pre-filled with NaN so unwritten elements show."""
     import torch
-    kpm, ui, kernel, info = build_kernel(config, kind)
+    kpm, ui, kernel, info = build_kernel(config, kind, hiprtc=hiprtc)
     ta, tc = kpm.dtypeTorch('A'), kpm.dtypeTorch('C')
     a_dev = to_device(SeededInputs.a_operand(a_mk, kpm.isATranspose), ta)
     b_dev = to_device(b_kn, ta)

@@ -1,7 +1,8 @@
 """Two fixed pseudo-random samples of tuning configs (both kernel families, all input types, both A
 layouts, prefetch flags, split-U, odd tile/wave shapes, 1..17 K tiles; the second with edge tiles in M,
 N and K), each checked bit for bit on small-integer data: the first against the CPU oracle, the second
-against the exact integer product.  The samples are deterministic, so the build step can precompile them."""
+against the exact integer product.  The samples are deterministic, so the build step can precompile them.
+Every sample runs twice: built by the hiprtc the process carries and by the system's (tests.gemm_helpers.hiprtc_params)."""
 import random
 
 import numpy as np
@@ -11,7 +12,7 @@ from codegendemo_amd import _native
 from codegendemo_amd.kcg import SeededInputs as SI
 from codegendemo_amd.kcg.ConfigGenerator import make_config
 from codegendemo_amd.kcg.Operators.matmul import kernelArgFromConfig
-from tests.gemm_helpers import run_gemm
+from tests.gemm_helpers import hiprtc_params, run_gemm
 
 pytestmark = pytest.mark.gpu
 
@@ -246,7 +247,8 @@ def random_odd_16bit_direct_configs(n=36, seed=20251127):
     return out
 
 
-def test_random_odd_16bit_shapes_through_the_direct_kernel_are_bit_exact():
+@pytest.mark.parametrize("hiprtc", hiprtc_params())
+def test_random_odd_16bit_shapes_through_the_direct_kernel_are_bit_exact(hiprtc):
     """fp16 / bf16 with odd extents: every other row of an operand starts 2 bytes off a 4-byte boundary, the chunk
     at the end of a row brings the next row's first elements with it, and the chunk at the end of the matrix is fetched
     from further down and moved into place in LDS."""
@@ -258,7 +260,7 @@ def test_random_odd_16bit_shapes_through_the_direct_kernel_are_bit_exact():
         a = SI.small_ints((M, K), SI.STREAM_A, lim=lim)
         b = SI.small_ints((K, N), SI.STREAM_B, lim=lim)
         print(f"[case] random odd 16-bit direct {i} {odd16_class(cfg)} {kernelArgFromConfig(cfg).values()}", flush=True)
-        got, info = run_gemm(cfg, a, b, kind)
+        got, info = run_gemm(cfg, a, b, kind, hiprtc=hiprtc)
         if info["lds_bytes"] == 0:
             direct += 1
             for c in odd16_class(cfg):
@@ -270,7 +272,8 @@ def test_random_odd_16bit_shapes_through_the_direct_kernel_are_bit_exact():
     assert direct >= 28 and all(classes.get(c, 0) >= 4 for c in ("a-kcont", "a-rowcont", "b", "k-odd")), (direct, classes)
 
 
-def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
+@pytest.mark.parametrize("hiprtc", hiprtc_params())
+def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact(hiprtc):
     cases = random_odd_direct_configs() + random_even_16bit_direct_configs()
     direct = 0
     for i, (cfg, kind) in enumerate(cases):
@@ -279,7 +282,7 @@ def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
         a = SI.small_ints((M, K), SI.STREAM_A, lim=lim)
         b = SI.small_ints((K, N), SI.STREAM_B, lim=lim)
         print(f"[case] random odd direct {i} {kernelArgFromConfig(cfg).values()}", flush=True)
-        got, info = run_gemm(cfg, a, b, kind)
+        got, info = run_gemm(cfg, a, b, kind, hiprtc=hiprtc)
         direct += int(info["lds_bytes"] == 0)
         want = a.astype(np.float64) @ b.astype(np.float64)
         bad = int((got.astype(np.float64) != want).sum()) + int(np.isnan(got).sum())
@@ -289,7 +292,8 @@ def test_random_odd_shapes_through_the_direct_kernel_are_bit_exact():
     assert direct >= 35
 
 
-def test_random_edge_config_sample_is_bit_exact():
+@pytest.mark.parametrize("hiprtc", hiprtc_params())
+def test_random_edge_config_sample_is_bit_exact(hiprtc):
     """Entries in {-1, 0, 1}: every sum is an integer of magnitude <= K, exact in fp32 and, for the 16-bit
     outputs (K <= 255 there), in fp16 and bf16 as well."""
     cases = random_edge_configs()
@@ -299,7 +303,7 @@ def test_random_edge_config_sample_is_bit_exact():
         a = SI.small_ints((M, K), SI.STREAM_A, lim=1)
         b = SI.small_ints((K, N), SI.STREAM_B, lim=1)
         print(f"[case] random edge {i} kind={kind} {kernelArgFromConfig(cfg).values()}", flush=True)
-        got, info = run_gemm(cfg, a, b, kind)
+        got, info = run_gemm(cfg, a, b, kind, hiprtc=hiprtc)
         direct += int(kind == _native.KIND_MFMA and info["lds_bytes"] == 0)
         want = a.astype(np.float64) @ b.astype(np.float64)
         bad = int((got.astype(np.float64) != want).sum()) + int(np.isnan(got).sum())
@@ -307,7 +311,8 @@ def test_random_edge_config_sample_is_bit_exact():
     assert direct >= 20
 
 
-def test_random_config_sample_is_bit_exact(oracle):
+@pytest.mark.parametrize("hiprtc", hiprtc_params())
+def test_random_config_sample_is_bit_exact(oracle, hiprtc):
     cases = random_configs()
     direct = 0
     for i, (cfg, kind) in enumerate(cases):
@@ -315,7 +320,7 @@ def test_random_config_sample_is_bit_exact(oracle):
         a = SI.small_ints((M, K), SI.STREAM_A, lim=2)
         b = SI.small_ints((K, N), SI.STREAM_B, lim=2)
         print(f"[case] random {i} kind={kind} {kernelArgFromConfig(cfg).values()}", flush=True)
-        got, info = run_gemm(cfg, a, b, kind)
+        got, info = run_gemm(cfg, a, b, kind, hiprtc=hiprtc)
         direct += int(kind == _native.KIND_MFMA and info["lds_bytes"] == 0)
         want = oracle.matmul(a, b, a_trans=False)
         bad = int((got != want).sum()) + int(np.isnan(got).sum())
