@@ -279,6 +279,28 @@ def compiler_identity():
     return buf.value.decode()
 
 
+class use_flags:
+    """Context manager: compiles inside it get `flags` (a string) as $KCG_EXTRA_FLAGS (None or "": none)."""
+
+    def __init__(self, flags):
+        self.flags = flags
+
+    def __enter__(self):
+        self.old = os.environ.get("KCG_EXTRA_FLAGS")
+        if self.flags:
+            os.environ["KCG_EXTRA_FLAGS"] = self.flags
+        else:
+            os.environ.pop("KCG_EXTRA_FLAGS", None)
+        return self
+
+    def __exit__(self, *exc):
+        if self.old is None:
+            os.environ.pop("KCG_EXTRA_FLAGS", None)
+        else:
+            os.environ["KCG_EXTRA_FLAGS"] = self.old
+        return False
+
+
 class use_hiprtc:
     """Context manager: compiles inside it use the hiprtc library at `path` (None: the process's own).  The
     library reads $KCG_HIPRTC_LIB at every compile and keeps such a compiler in a link namespace of its own."""

@@ -6,6 +6,12 @@
 
 namespace kcg {
 
+// Every lambda of this file is inlined by attribute.  The K loop is a forest of small generic lambdas (static_for
+// bodies, one instantiation per tile, k-step, row and slot: thousands of functions); left to the optimiser's inliner
+// they are inlined just the same, but only after argument promotion, attribute inference and the inliner's cost model
+// have looked at each of them, which took most of the compile time of the large tiles.
+#define KCG_INL __attribute__((always_inline))
+
 // ---------------------------------------------------------------------------------------------
 // In-kernel time line (diagnostic build, -DKCG_TIMELINE=1 or 2 through $KCG_EXTRA_FLAGS; 0 = off, no
 // code).  Every wave of gemm_mfma_direct then writes one record of KCG_TL_WORDS 64-bit words to the buffer
@@ -25,8 +31,8 @@ namespace kcg {
 #endif
 // Diagnostic builds only (never set by the library itself; C is then WRONG): the K loop of the direct-staging
 // kernel without its global->LDS fetches (the stages keep the first tiles, which the prologue still fetches)
-// resp. without its fragment reads (the matrix-core instructions keep running on the first fragments).
-// Timing such builds shows what each part of the data movement costs a launch.
+// resp. without its fragment reads (the matrix-core instructions keep running on the first fragments; 1: no fragment
+// reads at all, 2: none of A, 3: none of B).  Timing such builds shows what each part of the data movement costs a launch.
 #ifndef KCG_DIAG_NO_FETCH
 #define KCG_DIAG_NO_FETCH 0
 #endif
@@ -104,6 +110,12 @@ struct StreamPlan {
   static constexpr int BW0 = RB * TNI;                             // B reads: slots [BW0, BW1)
   static constexpr int BW1 = DA > 1 ? (TMI - 1) * TNI : NM;
   static constexpr int slot_b(int j) { return BW0 + (j * (BW1 - BW0)) / TNI; }
+  // (non-decreasing in j: the B fragments read behind slot q of a step are the range [first_b(q), first_b(q + 1)))
+  static constexpr int first_b(int q) {
+    int j = 0;
+    while (j < TNI && slot_b(j) < q) ++j;
+    return j;
+  }
   // issue times in half slots: a row's A read comes first in its slot, a B read follows the
   // matrix-core instruction of its slot
   static constexpr int time_a(int step, int row) { return (step * NM + (row - DA) * TNI) * 2; }
@@ -126,6 +138,23 @@ struct StreamPlan {
       }
     }
     return cmin(n, 15);                                            // the counter field has 4 bits; less is safe
+  }
+};
+
+// Where on the time line of the K loop the NFETCH fetch instructions of a K tile are issued: item f behind the
+// matrix-core instruction of slot pos(f), counted from the start of the tile that begins the fetch (a position of MT or
+// more lies in the next tile).  pos is non-decreasing in f: the items of a slot are the range [lo(q), lo(q + 1)).
+template <int NFETCH, int NIA, int BAR, int SPREAD>
+struct FetchSlots {
+  static constexpr int pos(int f) { return BAR + (f * SPREAD) / NFETCH; }
+  static constexpr int lo(int q) {                                  // the first item whose position is q or later
+    int f = 0;
+    while (f < NFETCH && pos(f) < q) ++f;
+    return f;
+  }
+  // (diagnostic builds: 1 drops every fetch of the K loop, 2 those of A only, 3 those of B only)
+  static constexpr bool on(int f) {
+    return KCG_DIAG_NO_FETCH == 0 || (KCG_DIAG_NO_FETCH == 2 && f >= NIA) || (KCG_DIAG_NO_FETCH == 3 && f < NIA);
   }
 };
 
@@ -159,7 +188,18 @@ struct DirectPlan {
   // (patch_final in the kernel).
   static constexpr int A_COLS = C::ATRANS ? C::M : C::K;          // row length of A as stored
   static constexpr int SH_A = (G - A_COLS % G) % G, SH_B = (G - C::N % G) % G;
-  static constexpr bool FIX_A = SH_A != 0, FIX_B = SH_B != 0;
+  // A straight from global memory into the fragment registers (-DKCG_A_GLOBAL=1; "AG" below): a k-contiguous A
+  // (IS_ATRANS=0) has the fragment layout of the matrix-core instructions in memory already - lane r + MF*g of a
+  // fragment wants the 16 bytes A[row r][k0 + G*g ...] - so one global_load_dwordx4 per lane and fragment delivers
+  // what the trip through LDS (a 1 KiB fetch into LDS + a ds_read_b128 per fragment) delivers, and the LDS that A
+  // occupied goes to more B stages.  Every wave then loads its own rows of A (the waves of one block row load
+  // the same ones).  Needs whole K tiles (no partial last tile: a fragment beyond K would read past a row).
+#ifndef KCG_A_GLOBAL
+#define KCG_A_GLOBAL 0
+#endif
+  static constexpr bool AG = KCG_A_GLOBAL != 0 && !C::ATRANS && C::K % C::BK == 0 && SPW > 0;
+  static constexpr int AG_DEPTH = 2;                              // k-steps an A fragment is loaded ahead of its use
+  static constexpr bool FIX_A = SH_A != 0 && !AG, FIX_B = SH_B != 0;
   static constexpr bool ELIGIBLE =
       (ES == 2 || (ES == 4 && sizeof(typename C::TC) == 4)) && C::SHMP && C::REGP && C::LC != 0 &&
       C::LSU == 1 && C::GLW_A == G && C::GLW_B == G &&
@@ -174,12 +214,14 @@ struct DirectPlan {
   // LDS stages: as many as fit in 160 KiB (or in half of it, see PAIR below), at most 4 (fetch distance =
   // NST-1 K tiles); an even number
   // when a tile is an odd number of k-steps (the B fragment double buffer alternates per step)
-  static constexpr int STAGE_BYTES = (C::BM + C::BN) * C::BK * ES;
+  static constexpr int A_STAGE_BYTES = AG ? 0 : C::BM * C::BK * ES;   // A's part of a stage (none when A bypasses LDS)
+  static constexpr int STAGE_BYTES = A_STAGE_BYTES + C::BN * C::BK * ES;
   static constexpr int NST_FIT = (160 * 1024) / STAGE_BYTES;
   // and no more than the fetch counter can tell apart: the wait for tile kt+1 allows the fetches of
-  // NST-2 younger tiles in flight, and that counter has 6 bits
-  static constexpr int NFETCH = ((C::BM + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
-  static constexpr int NST_VM = 2 + 63 / (NFETCH > 0 ? NFETCH : 1);
+  // NST-2 younger tiles in flight (and, with AG, the A loads issued in that time), and that counter has 6 bits
+  static constexpr int NFETCH = (((AG ? 0 : C::BM) + C::BN) * C::BK / G) / (64 * (NW > 0 ? NW : 1));   // per wave and tile
+  static constexpr int VMOPS = NFETCH + (AG ? SPW * (WM / MF) : 0);                                    // ... all counted operations
+  static constexpr int NST_VM = 2 + 63 / (VMOPS > 0 ? VMOPS : 1);
   static constexpr int NST_MAX = NST_FIT < NST_VM ? NST_FIT : NST_VM;
   // Two blocks on a compute unit beat one block with deeper staging when the launch has more blocks than the
   // chip has compute units (C::NUM_CU): one block's prologue, barrier waits and C stores run under the other's
@@ -274,11 +316,92 @@ struct FetchMap {
     const bool moved = P::FIX_B && last_tile && k == kvalid - 1 && n0 + n + G > N;
     return Src{(k * N + n - (moved ? P::SH_B : 0)) * ES, moved};
   }
+  // DirectPlan::AG: A fragments come straight from global memory.  The waves of wave row wy of the block at row m0
+  // read from row ag_row0 of the block tile on (a wave whose rows all lie beyond M: from the last row that exists, so
+  // that the lanes' offsets from there, unsigned 32-bit values, are never negative); for row block i of its fragments
+  // a lane reads the 16 bytes at ag_lane from there (+ the k-step's KS elements): row i*MF + lane%MF (rows beyond M:
+  // the last row; their results are not stored), k values G*(lane/MF) ...
+  __host__ __device__ static int ag_row0(int wy, int m0) {
+    int r = wy * P::WM;
+    if constexpr (EDGE_M) r = cmin(r, M - 1 - m0);
+    return r;
+  }
+  __host__ __device__ static unsigned ag_lane(int i, int lane, int m0, int row0) {
+    int row = i * P::MF + lane % P::MF;
+    if constexpr (EDGE_M) row = cmin(row, M - 1 - m0 - row0);
+    return (unsigned)((row * K + G * (lane / P::MF)) * ES);
+  }
   // byte offset of a block's tile kt from the start of A / B
   static constexpr long A_KT_BYTES = AK ? (long)BK * ES : (long)BK * M * ES;   // one K tile further
   static constexpr long B_KT_BYTES = (long)BK * N * ES;
   __host__ __device__ static constexpr long a_tile(int m0, int kt) { return (AK ? (long)m0 * K : (long)m0) * ES + kt * A_KT_BYTES; }
   __host__ __device__ static constexpr long b_tile(int n0, int kt) { return (long)n0 * ES + kt * B_KT_BYTES; }
+};
+
+// Order in which a wave of the direct-staging kernel issues the operations its vector-memory counter (vmcnt) counts
+// when A bypasses LDS (DirectPlan::AG): the global->LDS fetches of B (NIB per K tile) and the A fragment loads (one per
+// row of matrix-core tiles and k-step, issued D k-steps ahead).  The counter retires in order, so "operation X has
+// completed" is "at most n operations issued after X are outstanding"; n is a property of this order, computed here at
+// compile time for every place the K loop waits.  The K loop must issue in exactly this order:
+//   prologue : B tiles 0..NPRO-1 | A steps 0..D-1
+//   tile t, slot q (= matrix-core instruction (s, i, j), q = s*NM + i*TNI + j), after the instruction:
+//              the B fetches whose position is q, ascending f (f of tile t+NST where pos(f) = q, f of tile t-1+NST
+//              where pos(f) - MT = q), then, if j = TNI-1 and that step exists, the A load of (step t*SPW+s+D, row i)
+template <int KTT, int SPW, int TMI, int TNI, int NIB, int NST, int BAR, int SPREAD, int D>
+struct VmSchedule {
+  static constexpr int NM = TMI * TNI, MT = SPW * NM, STEPS = KTT * SPW;
+  static constexpr int NPRO = cmin(NST, KTT);
+  static constexpr int PRO_A_STEPS = cmin(D, STEPS);
+  static constexpr int PRO_OPS = NPRO * NIB + PRO_A_STEPS * TMI;
+  static constexpr bool hn(int t) { return t + NST < KTT; }                              // tile t begins the fetch of tile t+NST
+  static constexpr bool hp(int t) { return t >= 1 && t - 1 + NST < KTT && SPREAD > MT - BAR; }   // ... completes that of tile t-1+NST
+  static constexpr int pos(int f) { return BAR + (f * SPREAD) / NIB; }                   // on the time line that starts at the issuing tile
+  static constexpr bool a_issued(int t, int s) { return t * SPW + s + D < STEPS; }
+  static constexpr int n_first() { int n = 0; for (int f = 0; f < NIB; ++f) n += pos(f) < MT ? 1 : 0; return n; }
+  static constexpr int ops_in_tile(int t) {
+    int n = (hn(t) ? n_first() : 0) + (hp(t) ? NIB - n_first() : 0);
+    for (int s = 0; s < SPW; ++s) n += a_issued(t, s) ? TMI : 0;
+    return n;
+  }
+  static constexpr int ops_in_slot(int t, int q) {
+    int n = (q % TNI == TNI - 1 && a_issued(t, q / NM)) ? 1 : 0;
+    for (int f = 0; f < NIB; ++f) n += ((hn(t) && pos(f) == q) ? 1 : 0) + ((hp(t) && pos(f) - MT == q) ? 1 : 0);
+    return n;
+  }
+  // operations issued before the matrix-core instruction of slot q of tile t (q = MT: all of the tile)
+  static constexpr int seq_at(int t, int q) {
+    int n = PRO_OPS;
+    for (int tt = 0; tt < t; ++tt) n += ops_in_tile(tt);
+    for (int qq = 0; qq < q; ++qq) n += ops_in_slot(t, qq);
+    return n;
+  }
+  // sequence number of the A load of (step gs, row i)
+  static constexpr int seq_a(int gs, int i) {
+    if (gs < D) return NPRO * NIB + gs * TMI + i;
+    const int t = (gs - D) / SPW, s = (gs - D) % SPW;
+    return seq_at(t, s * NM + i * TNI + TNI) - 1;                                        // the last operation of the row's last slot
+  }
+  // a sequence number by which every B fetch of tile u has been issued (the last operation of the slot of its last fetch)
+  static constexpr int seq_b_done(int u) {
+    if (u < NPRO) return (u + 1) * NIB - 1;
+    const int p = pos(NIB - 1);
+    return p < MT ? seq_at(u - NST, p + 1) - 1 : seq_at(u - NST + 1, p - MT + 1) - 1;
+  }
+  static constexpr int clamp(int n) { return n < 0 ? 0 : (n > 63 ? 63 : n); }
+  // operations that may be outstanding when row i of step s of tile t starts (its A fragment has arrived) ...
+  static constexpr int wait_a(int t, int s, int i) { return clamp(seq_at(t, s * NM + i * TNI) - 1 - seq_a(t * SPW + s, i)); }
+  // ... and at the barrier of tile t (slot BAR of it has not been issued; tile t+1 has landed)
+  static constexpr int wait_b(int t) { return clamp(seq_at(t, BAR) - 1 - seq_b_done(t + 1)); }
+  // at the end of the prologue: B tile 0 has landed
+  static constexpr int wait_pro() { return clamp(PRO_OPS - 1 - seq_b_done(0)); }
+  // tiles t0 and t1 wait with the same counts everywhere (they can share their code)
+  static constexpr bool same_waits(int t0, int t1) {
+    if (wait_b(t0) != wait_b(t1)) return false;
+    for (int s = 0; s < SPW; ++s)
+      for (int i = 0; i < TMI; ++i)
+        if (wait_a(t0, s, i) != wait_a(t1, s, i) || a_issued(t0, s) != a_issued(t1, s)) return false;
+    return true;
+  }
 };
 
 template <class C>
@@ -303,8 +426,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int ES = P::ES, G = P::G;                   // element size; elements per 16-byte chunk
   constexpr int CHK = BK / G;                           // chunks per row of a k-contiguous tile
   constexpr int NCHA = BM / G, NCHB = BN / G;           // chunks per row of a row-contiguous tile
-  constexpr int A_BYTES = BM * BK * ES, B_BYTES = BN * BK * ES, STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int NIA = FM::NIA, NIB = FM::NIB;           // fetch instructions per wave and tile
+  constexpr bool AG = P::AG;                            // A goes from global memory straight into the fragment registers
+  constexpr int A_BYTES = P::A_STAGE_BYTES, B_BYTES = BN * BK * ES, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int NIA = AG ? 0 : FM::NIA, NIB = FM::NIB;  // fetch instructions per wave and tile
   constexpr int FETCH_BYTES = 64 * 16;                  // LDS bytes one fetch instruction of a wave fills
   typedef Mfma<T, MF> MI;
   typedef typename MI::Acc Acc;
@@ -333,38 +457,42 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   constexpr int NST = P::NST;
   __shared__ __attribute__((aligned(1024))) char lds_all[NST * STAGE_BYTES];
   (void)smem;
-  auto stage_ptr = [&](auto stage_c) -> char* { return lds_all + decltype(stage_c)::value * STAGE_BYTES; };
+  auto stage_ptr = [&](auto stage_c) KCG_INL -> char* { return lds_all + decltype(stage_c)::value * STAGE_BYTES; };
 
-  auto swz_n = [](int k, int nch) { return FM::swz_n(k, nch); };
+  auto swz_n = [](int k, int nch) KCG_INL { return FM::swz_n(k, nch); };
 
   // ---- fetch: global -> LDS ------------------------------------------------------------------
   // Address = scalar tile base (advances with kt) + a 32-bit byte offset per lane and fetch item that
   // never changes (FetchMap): the K loop spends no vector instruction on addresses.
-  auto off_a = [&](int idx) -> unsigned { return (unsigned)FM::a(wave, lane, idx, m0, BK, false).off; };
-  auto off_b = [&](int j) -> unsigned { return (unsigned)FM::b(wave, lane, j, n0, BK, false).off; };
-  unsigned voff_a[NIA], voff_b[NIB];
+  auto off_a = [&](int idx) KCG_INL -> unsigned { return (unsigned)FM::a(wave, lane, idx, m0, BK, false).off; };
+  auto off_b = [&](int j) KCG_INL -> unsigned { return (unsigned)FM::b(wave, lane, j, n0, BK, false).off; };
+  unsigned voff_a[NIA > 0 ? NIA : 1], voff_b[NIB];
 #pragma unroll
   for (int idx = 0; idx < NIA; ++idx) voff_a[idx] = off_a(idx);
 #pragma unroll
   for (int j = 0; j < NIB; ++j) voff_b[j] = off_b(j);
-  const char* const a_base = (const char*)A + FM::a_tile(m0, 0);
+  // AG: every wave reads its own WM rows of A, from ag_row0 on.  A wave whose rows all lie beyond M starts at the
+  // last row that exists, so that the per-lane offsets from there (unsigned 32-bit) never have to be negative.
+  const int ag_row0 = FM::ag_row0(wy, m0);
+  const char* const a_base = (const char*)A + FM::a_tile(m0, 0) + (AG ? (long)ag_row0 * K * ES : 0L);
   const char* const b_base = (const char*)B + FM::b_tile(n0, 0);
   constexpr long A_KT_BYTES = FM::A_KT_BYTES, B_KT_BYTES = FM::B_KT_BYTES;   // one K tile further
   // The tile bases pass through an empty asm: the compiler must not fold the per-tile scalar part
   // into the per-lane part (it would hoist "base + lane offset" as a 64-bit vector value and add the
   // tile offset with vector instructions); kept apart, the fetch uses its scalar-base addressing form.
   struct TileBase { const char* a; const char* b; };
-  auto tile_base = [&](int kt) {
+  auto tile_base = [&](int kt) KCG_INL {
     if constexpr (KCG_DIAG_FETCH_TILE0 != 0) kt = 0;
     TileBase t = {a_base + kt * A_KT_BYTES, b_base + kt * B_KT_BYTES};
     asm("" : "+s"(t.a), "+s"(t.b));
     return t;
   };
   // partial_c: the tile fetched is the last one and FINAL_SPECIAL
-  auto fetch_item = [&](int idx, const TileBase& tb, auto stage_c, auto partial_c) {
+  auto fetch_item = [&](auto idx_c, const TileBase& tb, auto stage_c, auto partial_c) KCG_INL {
     constexpr bool PARTIAL = decltype(partial_c)::value;
+    constexpr int idx = decltype(idx_c)::value;
     char* st = stage_ptr(stage_c);
-    if (idx < NIA) {
+    if constexpr (idx < NIA) {
       long off;
       if constexpr (PARTIAL) off = FM::a(wave, lane, idx, m0, KLAST, true).off;   // (signed: a moved chunk may start in front of the tile base)
       else {
@@ -375,7 +503,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(st + FETCH_BYTES * (wave * NIA + idx)), 16, 0, KCG_FETCH_AUX);
     } else {
-      const int j = idx - NIA;
+      constexpr int j = idx - NIA;
       long off;
       if constexpr (PARTIAL) off = FM::b(wave, lane, j, n0, KLAST, true).off;
       else {
@@ -393,9 +521,9 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // upper part then stands for does not exist: columns beyond N, rows beyond M or k values beyond K).
   // Called by every wave once its own fetches of the last tile have landed, in front of the barrier that
   // publishes the tile.
-  auto patch_final = [&](auto stage_c) {
+  auto patch_final = [&](auto stage_c) KCG_INL {
     const unsigned st = (unsigned)(unsigned long)stage_ptr(stage_c);
-    auto shift_down = [&](unsigned addr, auto bytes_c) {
+    auto shift_down = [&](unsigned addr, auto bytes_c) KCG_INL {
       constexpr int SB = decltype(bytes_c)::value, WS = SB / 4, BS = (SB % 4) * 8;   // whole words; bits inside a word
       u32x4 w;
       asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(w) : "v"(addr) : "memory");
@@ -496,7 +624,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   //   32-bit: one 32-bit read per k value.
   // The swizzle of a row depends on the lane only (swz_n looks at k bits that s and the read number do
   // not change).
-  auto rc_lane_base = [&](int toff, int nch, int rowbase) {
+  auto rc_lane_base = [&](int toff, int nch, int rowbase) KCG_INL {
     if constexpr (ES == 2) {
       const int n = rowbase + 16 * tsub + 4 * (tx % 4);
       const int k = 8 * fgrp + tx / 4;
@@ -510,9 +638,13 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   unsigned b_lane[TNI];
 #pragma unroll
   for (int j = 0; j < TNI; ++j) b_lane[j] = rc_lane_base(A_BYTES, NCHB, wx * WN + j * MF);
-  constexpr int NALANE = AK ? SPW : TMI;
+  constexpr int NALANE = AG ? TMI : (AK ? SPW : TMI);
   unsigned a_lane[NALANE];
-  if constexpr (AK) {
+  if constexpr (AG) {
+    // byte offset of the lane's 16 bytes of fragment row block i from the wave's part of the K tile
+#pragma unroll
+    for (int i = 0; i < TMI; ++i) a_lane[i] = FM::ag_lane(i, lane, m0, ag_row0);
+  } else if constexpr (AK) {
 #pragma unroll
     for (int st = 0; st < SPW; ++st)
       a_lane[st] = lds0 + (unsigned)(LK::slot(wy * WM + frow, st * KH + fgrp) * 16);   // swizzle: row%16 = frow%16 only
@@ -520,8 +652,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
 #pragma unroll
     for (int i = 0; i < TMI; ++i) a_lane[i] = rc_lane_base(0, NCHA, wy * WM + i * MF);
   }
-  auto split_base = [](unsigned lane_base, int imm) { return lane_base + (unsigned)(imm / 65536) * 65536u; };
-  auto read_rc = [&](unsigned lane_base, auto imm_c, auto nch_c, FragRc* dst) {
+  auto split_base = [](unsigned lane_base, int imm) KCG_INL { return lane_base + (unsigned)(imm / 65536) * 65536u; };
+  auto read_rc = [&](unsigned lane_base, auto imm_c, auto nch_c, FragRc* dst) KCG_INL {
     constexpr int IMM0 = decltype(imm_c)::value, ROW = decltype(nch_c)::value * 16;   // bytes per tile row
     if constexpr (ES == 2) {
       constexpr int IMM1 = IMM0 + 4 * ROW;                              // second block: four rows further
@@ -539,7 +671,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     }
   };
   // fragment f of k-step s of the stage: s, f and the stage are compile-time constants (IntC)
-  auto load_a = [&](auto stage_c, auto s_c, auto f_c, FragA* dst) {
+  auto load_a = [&](auto stage_c, auto s_c, auto f_c, FragA* dst) KCG_INL {
     constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
     if constexpr (AK) {
       constexpr int IMM = ST * STAGE_BYTES + F * MF * CHK * 16;
@@ -549,20 +681,27 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
       read_rc(a_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHA * 16>(), IntC<NCHA>(), dst);
     }
   };
-  auto load_b = [&](auto stage_c, auto s_c, auto f_c, FragB* dst) {
+  // AG: fragment f of k-step s of the K tile at `base` (scalar), straight from global memory.  Like the LDS reads
+  // an instruction the compiler does not see as a load: the K loop waits for it itself (VmSchedule).
+  auto load_ag = [&](const char* base, auto s_c, auto f_c, FragLd* dst) KCG_INL {
+    constexpr int S = decltype(s_c)::value, F = decltype(f_c)::value;
+    const unsigned off = a_lane[F];
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst->q) : "v"(off), "s"(base), "n"(S * KS * ES));
+  };
+  auto load_b = [&](auto stage_c, auto s_c, auto f_c, FragB* dst) KCG_INL {
     constexpr int ST = decltype(stage_c)::value, S = decltype(s_c)::value, F = decltype(f_c)::value;
     read_rc(b_lane[F], IntC<ST * STAGE_BYTES + S * KS * NCHB * 16>(), IntC<NCHB>(), dst);
   };
   // lgkmcnt(0): every LDS read issued so far has returned
-  auto wait_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
+  auto wait_lds = [&]() KCG_INL { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
 
   // prologue, first half: the first NST tiles go out together (the wait further down is for tile 0
   // alone: its successors' memory latency overlaps with it instead of following it), and before
   // anything else that takes time: clearing the accumulators runs under that latency
-  static_for<0, NST>([&](auto t) {
-    if (decltype(t)::value < KTT) {
-#pragma unroll
-      for (int i = 0; i < NFETCH; ++i) fetch_item(i, tile_base(decltype(t)::value), t, BoolC<(FINAL_SPECIAL && decltype(t)::value == KTF)>());
+  static_for<0, NST>([&](auto t) KCG_INL {
+    if constexpr (decltype(t)::value < KTT) {
+      const TileBase tb = tile_base(decltype(t)::value);
+      static_for<0, NFETCH>([&](auto i) KCG_INL { fetch_item(i, tb, t, BoolC<(FINAL_SPECIAL && decltype(t)::value == KTF)>()); });
     }
   });
 
@@ -600,7 +739,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // (the further ahead, the earlier the barrier stands in the last step and the more room the fetches
   // behind it have; measured best at the maximum)
   constexpr int DA = cmax(1, cmin(TMI - 1, KCG_SCHED_A_AHEAD > 0 ? KCG_SCHED_A_AHEAD : TMI - 1));
-  typedef StreamPlan<TMI, TNI, DA, (AK ? 1 : RC_READS), RC_READS> SP;
+  typedef StreamPlan<TMI, TNI, DA, (AG ? 0 : AK ? 1 : RC_READS), RC_READS> SP;
   constexpr int RB = SP::RB;
   constexpr int MT = SPW * NM;
   constexpr int BAR = (SPW - 1) * NM + RB * TNI;
@@ -608,16 +747,31 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   static_assert(TMI >= 2, "the streaming schedule needs two rows of matrix-core tiles per wave");
   static_assert((NST * SPW) % 2 == 0, "B double buffer: the parity of a step must follow from its stage");
   // s_waitcnt vmcnt(n), everything else unconstrained: n fetches of this wave may still be in flight
-  static_assert((NST - 2) * NFETCH < 64, "vmcnt has 6 bits");
-  auto vmcnt_only = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
-  auto tiles_ahead = [](int t) {
+  static_assert((NST - 2) * P::VMOPS < 64, "vmcnt has 6 bits");
+  constexpr int SPREAD = NST >= 3 ? MT : TAIL;                            // see "One K tile" below
+  constexpr int AGD = P::AG_DEPTH;
+  typedef VmSchedule<KTT, SPW, TMI, TNI, NIB, NST, BAR, SPREAD, AGD> VS;  // AG only
+  static_assert(!AG || ((NST * SPW) % AGD == 0 && KR == 0), "AG: the ring slot of a fragment must follow from stage and step");
+  auto vmcnt_only = [](int n) KCG_INL { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
+  auto tiles_ahead = [](int t) KCG_INL {
     const int last = cmin(KTT - 1, t == 0 ? NST - 1 : t - 1 + NST);  // newest tile whose fetch has been issued
     return cmax(0, last - (t + 1));
   };
 
   // prologue, second half
   constexpr int NPRO = cmin(NST, KTT);                                    // tiles the prologue has issued
-  __builtin_amdgcn_s_waitcnt(vmcnt_only(cmin(63, (NPRO - 1) * NFETCH)));  // this wave's chunks of tile 0 are in LDS
+  // AG: A fragments live in a ring of AGD k-steps, fa[(step % AGD) * TMI + row]; the first AGD steps are loaded here
+  FragA fa[AG ? AGD * TMI : TMI];
+  if constexpr (AG) {
+    static_for<0, cmin(AGD, KTT * SPW)>([&](auto gs_c) KCG_INL {
+      constexpr int GS = decltype(gs_c)::value;
+      const TileBase tb = tile_base(GS / SPW);
+      static_for<0, TMI>([&](auto i) KCG_INL { load_ag(tb.a, IntC<GS % SPW>(), i, &fa[(GS % AGD) * TMI + decltype(i)::value]); });
+    });
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(VS::wait_pro()));
+  } else {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(cmin(63, (NPRO - 1) * NFETCH)));  // this wave's chunks of tile 0 are in LDS
+  }
   asm volatile("" ::: "memory");
   if constexpr ((P::FIX_A || P::FIX_B) && KTT == 1) patch_final(IntC<0>());
   __builtin_amdgcn_s_barrier();                                            // ... and everyone's (bare barrier: see the K loop)
@@ -626,12 +780,14 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   tl[1] = tl_realtime();
   const unsigned long long tl_c0 = tl_cycles();
 #endif
-  FragA fa[TMI];
   FragB fb[2][TNI];
-  static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
-  static_for<0, (KCG_DIAG_NO_LDS_READS ? TMI : DA)>([&](auto i) { load_a(IntC<0>(), IntC<0>(), i, &fa[decltype(i)::value]); });
-  if constexpr (KCG_DIAG_NO_LDS_READS != 0 && SPW > 1)
-    static_for<0, TNI>([&](auto j) { load_b(IntC<0>(), IntC<1>(), j, &fb[1][decltype(j)::value]); });
+  constexpr bool NO_READS_A = KCG_DIAG_NO_LDS_READS == 1 || KCG_DIAG_NO_LDS_READS == 2;   // diagnostic builds
+  constexpr bool NO_READS_B = KCG_DIAG_NO_LDS_READS == 1 || KCG_DIAG_NO_LDS_READS == 3;
+  static_for<0, TNI>([&](auto j) KCG_INL { load_b(IntC<0>(), IntC<0>(), j, &fb[0][decltype(j)::value]); });
+  if constexpr (!AG)
+    static_for<0, (NO_READS_A ? TMI : DA)>([&](auto i) KCG_INL { load_a(IntC<0>(), IntC<0>(), i, &fa[decltype(i)::value]); });
+  if constexpr (NO_READS_B && SPW > 1)
+    static_for<0, TNI>([&](auto j) KCG_INL { load_b(IntC<0>(), IntC<1>(), j, &fb[1][decltype(j)::value]); });
   wait_lds();   // the counted waits of the loop assume that nothing older than its own reads is in flight
 
   // One K tile.  CUR: the stage it computes from; H1: tile kt+1 exists; HN: tile kt+NST exists; HP: the
@@ -643,8 +799,12 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   // instructions are spread over the whole period up to the next barrier (the memory pipeline of a CU
   // takes 16 cycles per 1 KiB fetch instruction; four waves issuing all of theirs right behind the
   // barrier would stall on it); with two stages they must all be issued in the rest of this tile.
-  constexpr int SPREAD = NST >= 3 ? MT : TAIL;
-  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c, auto ns_c, auto pn_c, auto pp_c, auto fixn_c) {
+  // AG: tsim_c is the tile's number in the operation order of VmSchedule (its own number, or for the tiles of the
+  // run-time loop that of the first tile that executes the same code).
+  typedef FetchSlots<NFETCH, NIA, BAR, SPREAD> FS;
+  auto tile = [&](int kt, auto cur_c, auto has1, auto hasn, auto hasp, auto ahead_c, auto ns_c, auto pn_c, auto pp_c, auto fixn_c,
+                  auto tsim_c) KCG_INL {
+    constexpr int TSIM = decltype(tsim_c)::value;
     constexpr int CUR = decltype(cur_c)::value, NS = decltype(ns_c)::value;
     constexpr int NXT = (CUR + 1) % NST, PRV = (CUR + NST - 1) % NST;
     constexpr bool H1 = decltype(has1)::value, HN = decltype(hasn)::value;
@@ -655,15 +815,23 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
     // the G consecutive k values that start at S*KS + G*(lane/MF); those of them that are >= K (what was
     // fetched in their place is arbitrary) are cleared before use.
     constexpr bool PARTIAL = KR > 0 && NS == SPWT && decltype(has1)::value == false && (KR % KS != 0);
-    static_for<0, NS>([&](auto s_c) {
+    static_for<0, NS>([&](auto s_c) KCG_INL {
       constexpr int S = decltype(s_c)::value;
       constexpr bool LAST = (S == NS - 1);
       constexpr bool MASK = PARTIAL && LAST;
       const int nvalid = KR - (S * KS + G * fgrp);   // how many of this lane's G consecutive k values lie below K
       constexpr int PB = (CUR * SPW + S) & 1;       // half of the B double buffer this step computes from
       constexpr bool NEXT = !LAST || H1;            // a next step exists, its fragments are read under this one
-      static_for<0, TMI>([&](auto i_c) {
+      constexpr int RING = AG ? ((CUR * SPW + S) % AGD) * TMI : 0;     // AG: this step's slots in the ring of A fragments
+      // AG: the load issued behind row I fetches row I of the step AGD further on, into the registers this row frees
+      constexpr bool A_NEXT = AG && (TSIM * SPW + S + AGD < KTT * SPW);
+      const char* a_next = nullptr;
+      if constexpr (A_NEXT) a_next = tile_base(kt + (S + AGD) / SPW).a;
+      static_for<0, TMI>([&](auto i_c) KCG_INL {
         constexpr int I = decltype(i_c)::value;
+        constexpr int FI = RING + I;
+        // AG: this row's A fragment has arrived (vmcnt counts fetches and A loads alike, in order)
+        if constexpr (AG) __builtin_amdgcn_s_waitcnt(vmcnt_only(VS::wait_a(TSIM, S, I)));
         // the fragments of this row have arrived.  Without a next step the reads the count relies on
         // are not issued: wait for everything instead.
         if constexpr (NEXT) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(SP::allowed(I)) : "memory");
@@ -675,7 +843,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           wait_lds();        // (level 2: the stamp's own wait must not count as barrier wait)
           const unsigned long long tl_b0 = tl_cycles();
 #endif
-          if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
+          if constexpr (H1 && AG) __builtin_amdgcn_s_waitcnt(vmcnt_only(VS::wait_b(TSIM)));
+          else if constexpr (H1) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(ahead_c)::value * NFETCH));
           wait_lds();        // this wave's reads of stage CUR have all returned
           if constexpr (decltype(fixn_c)::value) patch_final(IntC<NXT>());   // tile kt+1 is the last one (nothing behind it in flight)
           // ... everyone's part; and every wave is done reading stage CUR.  The bare barrier instruction:
@@ -694,7 +863,7 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         }
         // the empty asm statements make the fragments "outputs" of the wait: the matrix-core
         // instructions that consume them cannot be scheduled in front of it
-        fa[I].pin();
+        fa[FI].pin();
         if constexpr (I == 0) {
 #pragma unroll
           for (int j = 0; j < TNI; ++j) fb[PB][j].pin();
@@ -702,8 +871,8 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
         if constexpr (MASK) {
           // (pinned again behind the selects: they must have been issued before the wait state that
           // separates them from the matrix-core instruction reading their results)
-          fa[I].keep_first(nvalid);
-          fa[I].pin();
+          fa[FI].keep_first(nvalid);
+          fa[FI].pin();
           if constexpr (I == 0) {
 #pragma unroll
             for (int j = 0; j < TNI; ++j) {
@@ -713,35 +882,41 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
           }
           asm volatile("s_nop 1" ::: "memory");
         }
-        if constexpr (KCG_DIAG_NO_LDS_READS != 0) {
+        if constexpr (NO_READS_A || AG) {
         } else if constexpr (I + DA < TMI) load_a(IntC<CUR>(), IntC<S>(), IntC<I + DA>(), &fa[I + DA]);
         else if constexpr (!LAST) load_a(IntC<CUR>(), IntC<S + 1>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
         else if constexpr (H1) load_a(IntC<NXT>(), IntC<0>(), IntC<I + DA - TMI>(), &fa[I + DA - TMI]);
-        static_for<0, TNI>([&](auto j_c) {
+        static_for<0, TNI>([&](auto j_c) KCG_INL {
           constexpr int J = decltype(j_c)::value;
           constexpr int slot = S * NM + I * TNI + J;
           // operands swapped (B fragment first): the accumulator then holds C^T tiles, i.e. each lane owns
           // one row m and groups of four consecutive n, which the epilogue stores as 128-bit vectors
           // odd rows run right to left: neighbours on the time line always share one operand
           constexpr int JC = (I & 1) ? TNI - 1 - J : J;
-          MI::run_tied(acc[I][JC], fb[PB][JC].get(), fa[I].get());
-          static_for<0, TNI>([&](auto jj_c) {
+          MI::run_tied(acc[I][JC], fb[PB][JC].get(), fa[FI].get());
+          static_for<SP::first_b(I * TNI + J), SP::first_b(I * TNI + J + 1)>([&](auto jj_c) KCG_INL {
             constexpr int JJ = decltype(jj_c)::value;
-            if constexpr (KCG_DIAG_NO_LDS_READS == 0 && SP::slot_b(JJ) == I * TNI + J) {
+            if constexpr (!NO_READS_B) {
               if constexpr (!LAST) load_b(IntC<CUR>(), IntC<S + 1>(), jj_c, &fb[PB ^ 1][JJ]);
               else if constexpr (H1) load_b(IntC<NXT>(), IntC<0>(), jj_c, &fb[PB ^ 1][JJ]);
             }
           });
-#pragma unroll
-          for (int f = 0; f < NFETCH; ++f) {
-            const int pos = BAR + (f * SPREAD) / NFETCH;          // position on the time line that starts at this tile
-            // (diagnostic builds: 1 drops every fetch of the K loop, 2 those of A only, 3 those of B only)
-            const bool fetch_on = KCG_DIAG_NO_FETCH == 0 || (KCG_DIAG_NO_FETCH == 2 && f >= NIA) || (KCG_DIAG_NO_FETCH == 3 && f < NIA);
-            if (fetch_on && HN && pos == slot) fetch_item(f, tbn, IntC<CUR>(), pn_c);
-            if (fetch_on && HP && pos - MT == slot) fetch_item(f, tbp, IntC<PRV>(), pp_c);
-          }
+          // the fetch items whose position on the time line (FetchSlots::pos, counted from the start of the tile that
+          // begins the fetch) is this slot: of tile kt+NST, and, a period later, of tile kt-1+NST; ascending f
+          if constexpr (HN)
+            static_for<FS::lo(slot), FS::lo(slot + 1)>([&](auto f_c) KCG_INL {
+              if constexpr (FS::on(decltype(f_c)::value)) fetch_item(f_c, tbn, IntC<CUR>(), pn_c);
+            });
+          if constexpr (HP)
+            static_for<FS::lo(slot + MT), FS::lo(slot + MT + 1)>([&](auto f_c) KCG_INL {
+              if constexpr (FS::on(decltype(f_c)::value)) fetch_item(f_c, tbp, IntC<PRV>(), pp_c);
+            });
           __builtin_amdgcn_sched_barrier(0);
         });
+        if constexpr (A_NEXT) {
+          load_ag(a_next, IntC<(S + AGD) % SPW>(), i_c, &fa[FI]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       });
     });
   };
@@ -752,21 +927,29 @@ __device__ __forceinline__ void gemm_mfma_direct(const typename C::TA* __restric
   typedef BoolC<false> No;
   constexpr bool FIX = P::FIX_A || P::FIX_B;
   tile(0, IntC<0>(), BoolC<(1 < KTT)>(), BoolC<(NST < KTT)>(), No(), IntC<tiles_ahead(0)>(), IntC<(0 < KT ? SPW : SPWT)>(),
-       BoolC<(FINAL_SPECIAL && NST == KTF)>(), No(), BoolC<(FIX && 2 == KTT)>());
-  constexpr int NFULL = KTF - NST - 1 > 0 ? KTF - NST - 1 : 0;   // tiles 1 .. KTF-NST-1 have kt+NST < KTF: ordinary tiles all round
-  constexpr int NG = NFULL / NST;
-  for (int g = 0; g < NG; ++g) {
-    static_for<0, NST>([&](auto sc) {
-      constexpr int S = decltype(sc)::value;
-      tile(1 + g * NST + S, IntC<(1 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>(), IntC<SPW>(), No(), No(), No());
-    });
-  }
-  static_for<1 + NG * NST, KTT>([&](auto tc) {
+       BoolC<(FINAL_SPECIAL && NST == KTF)>(), No(), BoolC<(FIX && 2 == KTT)>(), IntC<0>());
+  auto static_tile = [&](auto tc) KCG_INL {
     constexpr int T = decltype(tc)::value;
     tile(T, IntC<T % NST>(), BoolC<(T + 1 < KTT)>(), BoolC<(T + NST < KTT)>(), BoolC<(T - 1 + NST < KTT)>(), IntC<tiles_ahead(T)>(),
          IntC<(T < KT ? SPW : SPWT)>(), BoolC<(FINAL_SPECIAL && T + NST == KTF)>(), BoolC<(FINAL_SPECIAL && T - 1 + NST == KTF)>(),
-         BoolC<(FIX && T + 2 == KTT)>());
-  });
+         BoolC<(FIX && T + 2 == KTT)>(), tc);
+  };
+  // The run-time loop starts at tile L0.  AG: the wait counts of a tile depend on what was issued up to NST-1
+  // tiles earlier, and the prologue issued the first NST tiles in another order than the loop does: the tiles in
+  // front of L0 = NST are unrolled with their own counts.
+  constexpr int L0 = AG ? cmax(NST, 2) : 1;
+  static_for<1, cmin(L0, KTT)>(static_tile);
+  constexpr int NFULL = KTF - NST - L0 > 0 ? KTF - NST - L0 : 0;   // tiles L0 .. KTF-NST-1 have kt+NST < KTF: ordinary tiles all round
+  constexpr int NG = NFULL / NST;
+  for (int g = 0; g < NG; ++g) {
+    static_for<0, NST>([&](auto sc) KCG_INL {
+      constexpr int S = decltype(sc)::value;
+      static_assert(!AG || NG == 0 || VS::same_waits(L0 + S, L0 + (NG > 0 ? NG - 1 : 0) * NST + S), "AG: the loop's tiles must wait alike");
+      tile(L0 + g * NST + S, IntC<(L0 + S) % NST>(), BoolC<true>(), BoolC<true>(), BoolC<true>(), IntC<NST - 2>(), IntC<SPW>(), No(), No(), No(),
+           IntC<L0 + S>());
+    });
+  }
+  static_for<cmax(L0, 1) + NG * NST, KTT>(static_tile);
 
   // the last matrix-core results must have left the pipeline before the epilogue reads them (the
   // compiler, which normally inserts these wait states, does not know the instructions above)

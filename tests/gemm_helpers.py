@@ -1,5 +1,7 @@
 """Shared helpers of the GPU parity tests: drive a config through the kcg API exactly the way the
 reference's tuner does (compile -> UserInputs -> CompiledKernelFactory -> CompiledKernel.run)."""
+import os
+
 import numpy as np
 
 from codegendemo_amd import _native
@@ -23,11 +25,11 @@ def hiprtc_params():
                          marks=pytest.mark.skipif(not os.path.exists(_native.SYSTEM_HIPRTC), reason="no system ROCm"))]
 
 
-def build_kernel(config, kind=_native.KIND_AUTO, device=0, hiprtc=None):
-    """hiprtc: path of the hiprtc library that compiles (None: the process's own)."""
+def build_kernel(config, kind=_native.KIND_AUTO, device=0, hiprtc=None, flags=None):
+    """hiprtc: path of the hiprtc library that compiles (None: the process's own); flags: extra compiler options."""
     kpm = kernelArgFromConfig(config)
     comp = KCGCompiler(kind=kind)
-    with _native.use_hiprtc(hiprtc):
+    with _native.use_hiprtc(hiprtc), _native.use_flags(flags or os.environ.get("KCG_EXTRA_FLAGS")):
         path, name, gx, gy, gz, bx, by, bz = comp.compileKernel(kpm)[0]
     ui = UserInputs(path, name, kpm)
     ui.m_gridDims = [gx, gy, gz]
@@ -42,11 +44,11 @@ def to_device(x, torch_dtype, device="cuda:0"):
     return torch.from_numpy(np.ascontiguousarray(x)).to(device=device, dtype=torch_dtype)
 
 
-def run_gemm(config, a_mk, b_kn, kind=_native.KIND_AUTO, poison=True, hiprtc=None):
+def run_gemm(config, a_mk, b_kn, kind=_native.KIND_AUTO, poison=True, hiprtc=None, flags=None):
     """a_mk: logical [M,K] fp32 numpy, b_kn: [K,N].  Returns (C as float64-free numpy in the config's
     C dtype upcast to fp32, info).  The output buffer is pre-filled with NaN so unwritten elements show."""
     import torch
-    kpm, ui, kernel, info = build_kernel(config, kind, hiprtc=hiprtc)
+    kpm, ui, kernel, info = build_kernel(config, kind, hiprtc=hiprtc, flags=flags)
     ta, tc = kpm.dtypeTorch('A'), kpm.dtypeTorch('C')
     a_dev = to_device(SeededInputs.a_operand(a_mk, kpm.isATranspose), ta)
     b_dev = to_device(b_kn, ta)

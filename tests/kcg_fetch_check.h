@@ -54,8 +54,26 @@ int main() {
           misaligned += (addr % 4) != 0;
           return 0;
         };
+        // A, read straight from global memory into fragment registers (DirectPlan::AG): every load of every lane
+        // stays inside A, and a lane whose row exists gets the 16 bytes of its row and k values
+        if constexpr (P::AG) {
+          for (int wy = 0; wy < Cfg::BLM; ++wy) {
+            const int row0 = F::ag_row0(wy, m0);
+            if (row0 < 0 || m0 + row0 >= M) return fail("AG: the wave's first row does not exist", by, bx, kt, wy, row0);
+            for (int st = 0; st < P::SPW; ++st)
+              for (int i = 0; i < P::WM / P::MF; ++i)
+                for (int lane = 0; lane < 64; ++lane) {
+                  const unsigned off = F::ag_lane(i, lane, m0, row0);
+                  const long addr = F::a_tile(m0, kt) + (long)row0 * K * ES + (long)(unsigned long)off + (long)st * P::KS * ES;
+                  if (addr < 0 || addr + 16 > a_bytes) return fail("AG load outside A", by, bx, kt, lane, addr);
+                  const int row = m0 + wy * P::WM + i * P::MF + lane % P::MF, kk = kt * BK + st * P::KS + G * (lane / P::MF);
+                  if (row < M && addr != ((long)row * K + kk) * ES) return fail("AG load is not the lane's fragment", by, bx, kt, lane, addr);
+                  ++chunks;
+                }
+          }
+        }
         // A
-        for (int r = 0; r < (F::AK ? BM : BK); ++r)
+        for (int r = 0; r < (P::AG ? 0 : F::AK ? BM : BK); ++r)
           for (int c = 0; c < (F::AK ? F::CHK : F::NCHA); ++c) {
             const int phys = F::AK ? F::LK::slot(r, c) : r * F::NCHA + (c ^ F::swz_n(r, F::NCHA));
             Got g;

@@ -46,8 +46,21 @@ def cases():
     return out
 
 
+def ag_cases():
+    """Shapes for the build that reads A straight from global memory (-DKCG_A_GLOBAL=1: A [M,K], whole K tiles):
+    full tiles, edge tiles in M and N, and block rows of which whole wave rows lie beyond M."""
+    out = []
+    for dtype, tile in TILES:
+        bm, bn, bk = tile["BM"], tile["BN"], tile["BK"]
+        for m, n, k in ((bm, bn, bk), (2 * bm, bn + 3, 3 * bk), (bm + 1, 2 * bn, 2 * bk), (bm - 1, bn, 5 * bk), (2 * bm - 17, bn - 1, 4 * bk),
+                        (bm // 2 - 1, bn, bk), (bm + bm // 4 + 2, bn, 2 * bk), (1, bn, 2 * bk), (3 * bm - bm // 2, 2 * bn - 8, 6 * bk)):
+            out.append(make_config(m, n, k, dtype=dtype, dtype_c=4, is_atrans=0, **tile, **DIRECT))
+    return out
+
+
 def run_check(job):
-    index, cfg, workdir = job
+    index, cfg, workdir = job[:3]
+    flags = list(job[3]) if len(job) > 3 else []
     values = kernelArgFromConfig(cfg).values()
     stub = _native.instantiation_source(values, _native.KIND_MFMA)
     if "DIRECT = true" not in stub:
@@ -57,7 +70,7 @@ def run_check(job):
     path = os.path.join(workdir, f"check_{index}")
     with open(path + ".hip", "w") as f:
         f.write(src)
-    p = subprocess.run([HIPCC, "--cuda-host-only", "-O1", "-std=c++17", "-include", "hip/hip_runtime.h", "-I", CSRC, "-I", HERE,
+    p = subprocess.run([HIPCC, "--cuda-host-only", "-O1", "-std=c++17", "-include", "hip/hip_runtime.h", "-I", CSRC, "-I", HERE] + flags + [
                         "-o", path, path + ".hip"], capture_output=True, text=True)
     if p.returncode:
         return index, "compile failed: " + p.stderr[-1500:]
@@ -77,3 +90,16 @@ def test_every_fetch_stays_inside_the_operands_and_lands_where_it_is_read(tmp_pa
         assert text.startswith("ok:"), f"case {index} (M, N, K, A layout, type, tile = {shape}): {text}"
         moved += int(text.split("chunks,")[1].split()[0])
     assert moved > 0          # the sample reaches the chunks at the end of a matrix
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_every_load_of_a_from_global_memory_stays_inside_a(tmp_path):
+    """The same walk for the build that loads A fragments straight from global memory: every lane's 16 bytes lie
+    inside A (also for waves whose rows all lie beyond M) and are the lane's row and k values where the row exists."""
+    jobs = [(i, cfg, str(tmp_path), ("-DKCG_A_GLOBAL=1",)) for i, cfg in enumerate(ag_cases())]
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        results = list(pool.map(run_check, jobs))
+    for index, text in results:
+        cfg = jobs[index][1]
+        shape = (cfg["M_SIZE"], cfg["N_SIZE"], cfg["K_SIZE"], cfg["DATATYPE_A"], cfg["BLOCK_SIZE_M"], cfg["BLOCK_SIZE_N"], cfg["BLOCK_SIZE_K"])
+        assert text.startswith("ok:"), f"case {index} (M, N, K, type, tile = {shape}): {text}"
