@@ -281,6 +281,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: first run a plain 256 MiB device copy three times, so that HBM counters "
                          "(FETCH_SIZE / WRITE_SIZE) of the same profiler run can be scaled by a kernel of known traffic")
+    ap.add_argument("--hiprtc", default="", help="path of the hiprtc library that builds the kernels (default: the one this "
+                    "process carries, i.e. the ROCm that PyTorch bundles); 'system' = /opt/rocm/lib/libhiprtc.so.7")
     ap.add_argument("--only-fp16", action="store_true",
                     help="profiling aid: run only the fp16 kernel (prints a reduced JSON line)")
     args = ap.parse_args()
@@ -292,6 +294,8 @@ def main():
     import torch
     from codegendemo_amd import _native
     _native.lib()   # raises if the native library is missing: there is no fallback
+    if args.hiprtc:
+        os.environ["KCG_HIPRTC_LIB"] = _native.SYSTEM_HIPRTC if args.hiprtc == "system" else args.hiprtc
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
@@ -312,7 +316,7 @@ def main():
         ms_step16, ms_launch16 = time_steps(kernel16, A16, B16, C16, args.steps, args.warmup)
         fl = 2.0 * kpm16.M * kpm16.N * kpm16.K
         print(json.dumps({"only": "fp16", "kernel": info16["kernel_name"], "launch_ms": ms_launch16,
-                          "tflops": fl / (ms_launch16 * 1e-3) / 1e12}))
+                          "tflops": fl / (ms_launch16 * 1e-3) / 1e12, "compiler": _native.compiler_identity()}))
         return
 
     # ---- preparation: every kernel built and loaded, every operand resident in HBM, before anything is timed.
@@ -357,7 +361,9 @@ def main():
                                + (", A stored [K,M]" if kpm.isATranspose else ", row-major A[M,K]")
                                + " B[K,N], uniform[-1,1) seeded, tuned config",
                    "kernel": info["kernel_name"], "kind": {1: "simt", 2: "mfma"}[info["kind"]],
-                   "lds_bytes": info["lds_bytes"], "grid": info["grid"][0], "block": info["block"][0]},
+                   "lds_bytes": info["lds_bytes"], "grid": info["grid"][0], "block": info["block"][0],
+                   "compiler": _native.compiler_identity(), "vgprs": info["vgprs"], "scratch_bytes": info["scratch_bytes"],
+                   "build_flags": info["build_flags"]},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS["f32"], "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS["f32"], "traffic": traffic32, "traffic_source": traffic32_note,
                      "launch_ms": ms_launch,
