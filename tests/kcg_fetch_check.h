@@ -10,12 +10,81 @@
 #pragma once
 #include <cstdio>
 
+// DirectPlan::AG: the wait counts of VmSchedule against an explicit list of the operations in the order the K loop issues
+// them (prologue: the B fetches of the first tiles, then the A loads of the first steps; per slot of a tile: the B fetches whose
+// position is that slot; behind a row's last slot: the A load of that row two steps on).  A wait for operation X with count n is
+// right if at most n operations were issued after X at that point; it is tight if exactly n were (or 63, the counter's limit).
+template <class P, class F>
+int check_vm_schedule() {
+  constexpr int SPW = P::SPW, TMI = P::WM / P::MF, TNI = P::WN / P::MF, NM = TMI * TNI, MT = SPW * NM;
+  constexpr int NST = P::NST, NIB = F::NIB, KTT = F::KTT, D = P::AG_DEPTH, STEPS = KTT * SPW;
+  constexpr int RB = 1, BAR = (SPW - 1) * NM + RB * TNI, SPREAD = NST >= 3 ? MT : MT - BAR;   // as in the kernel (A_AHEAD at its default)
+  typedef kcg::VmSchedule<KTT, SPW, TMI, TNI, NIB, NST, BAR, SPREAD, D> VS;
+  struct Op { int is_a, x, y; };                         // A load of (step x, row y) or B fetch of (tile x, item y)
+  static Op ops[1 << 20];
+  int n = 0;
+  auto last_of = [&](int is_a, int x, int y) {           // index of that operation, -1 if it was never issued
+    for (int k = n - 1; k >= 0; --k)
+      if (ops[k].is_a == is_a && ops[k].x == x && (y < 0 || ops[k].y == y)) return k;
+    return -1;
+  };
+  auto bad = [](const char* what, int t, int s, int i, int have, int allowed) {
+    printf("FAILED: vm schedule: %s (tile %d, step %d, row %d): waits with %d, %d operations were issued behind it\n", what, t, s, i, have, allowed);
+    return 1;
+  };
+  long loose = 0;
+  const int npro = NST < KTT ? NST : KTT;
+  for (int t = 0; t < npro; ++t)
+    for (int f = 0; f < NIB; ++f) ops[n++] = Op{0, t, f};
+  for (int gs = 0; gs < (D < STEPS ? D : STEPS); ++gs)
+    for (int i = 0; i < TMI; ++i) ops[n++] = Op{1, gs, i};
+  {
+    const int allowed = n - 1 - last_of(0, 0, -1);
+    if (VS::wait_pro() > allowed) return bad("B tile 0 at the end of the prologue", 0, 0, 0, VS::wait_pro(), allowed);
+  }
+  for (int t = 0; t < KTT; ++t)
+    for (int s = 0; s < SPW; ++s)
+      for (int i = 0; i < TMI; ++i) {
+        const int ia = last_of(1, t * SPW + s, i);
+        if (ia < 0) return bad("an A fragment that was never loaded", t, s, i, 0, 0);
+        const int allowed_a = n - 1 - ia < 63 ? n - 1 - ia : 63;
+        if (VS::wait_a(t, s, i) > allowed_a) return bad("A fragment", t, s, i, VS::wait_a(t, s, i), allowed_a);
+        loose += allowed_a - VS::wait_a(t, s, i);
+        if (s == SPW - 1 && i == RB && t + 1 < KTT) {
+          int ib = -1;
+          for (int f = 0; f < NIB; ++f) {
+            const int k = last_of(0, t + 1, f);
+            if (k < 0) return bad("a B fetch of the next tile that was never issued", t, s, f, 0, 0);
+            ib = k > ib ? k : ib;
+          }
+          const int allowed_b = n - 1 - ib < 63 ? n - 1 - ib : 63;
+          if (VS::wait_b(t) > allowed_b) return bad("B tile at the barrier", t, s, i, VS::wait_b(t), allowed_b);
+          if (allowed_b - VS::wait_b(t) > NIB) return bad("B tile at the barrier waits for far more than it needs", t, s, i, VS::wait_b(t), allowed_b);
+        }
+        for (int j = 0; j < TNI; ++j) {
+          const int q = s * NM + i * TNI + j;
+          for (int f = 0; f < NIB; ++f) {
+            const int pos = BAR + (f * SPREAD) / NIB;
+            if (t + NST < KTT && pos == q) ops[n++] = Op{0, t + NST, f};
+            if (t >= 1 && t - 1 + NST < KTT && SPREAD > MT - BAR && pos - MT == q) ops[n++] = Op{0, t - 1 + NST, f};
+          }
+        }
+        if (t * SPW + s + D < STEPS) ops[n++] = Op{1, t * SPW + s + D, i};
+        if (n > (1 << 20) - 64) return bad("too many operations for this check", t, s, i, n, 0);
+      }
+  if (loose != 0) return bad("A waits are not tight: summed slack", 0, 0, 0, (int)loose, 0);
+  return 0;
+}
+
 int main() {
   typedef kcg::DirectPlan<Cfg> P;
   typedef kcg::FetchMap<Cfg> F;
   if (!P::OK) {
     printf("not a direct-staging instantiation\n");
     return 2;
+  }
+  if constexpr (P::AG) {
+    if (check_vm_schedule<P, F>()) return 1;
   }
   constexpr int M = F::M, N = F::N, K = F::K, BM = F::BM, BN = F::BN, BK = F::BK, G = F::G, ES = F::ES, NW = F::NW;
   const long a_bytes = (long)M * K * ES, b_bytes = (long)K * N * ES;

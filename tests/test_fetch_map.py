@@ -95,7 +95,10 @@ def test_every_fetch_stays_inside_the_operands_and_lands_where_it_is_read(tmp_pa
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 def test_every_load_of_a_from_global_memory_stays_inside_a(tmp_path):
     """The same walk for the build that loads A fragments straight from global memory: every lane's 16 bytes lie
-    inside A (also for waves whose rows all lie beyond M) and are the lane's row and k values where the row exists."""
+    inside A (also for waves whose rows all lie beyond M) and are the lane's row and k values where the row exists.
+    The checker also lists the counted memory operations of a wave in the order the K loop issues them and
+    compares every wait count of the kernel's compile-time schedule (VmSchedule) with it: no wait may allow more
+    operations in flight than were issued behind the one it waits for, and the waits for A fragments are exact."""
     jobs = [(i, cfg, str(tmp_path), ("-DKCG_A_GLOBAL=1",)) for i, cfg in enumerate(ag_cases())]
     with ThreadPoolExecutor(max_workers=8) as pool:
         results = list(pool.map(run_check, jobs))
