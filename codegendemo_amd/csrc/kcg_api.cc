@@ -690,7 +690,9 @@ static int build_variant(const kcg::MatmulConfig& c, int k, bool allow_direct, c
   }
   if (diagnostic) {
     out->build_flags |= KCG_BUILD_DIAGNOSTIC;
-    note = "note: diagnostic build (" + std::string(getenv("KCG_EXTRA_FLAGS")) + "): the result of this kernel is wrong on purpose";
+    std::string given;
+    for (const auto& f : extra) given += (given.empty() ? "" : " ") + f;
+    note = "note: diagnostic build (" + given + "): the result of this kernel is wrong on purpose";
   }
   if (declined) out->build_flags |= KCG_BUILD_DIRECT_DECLINED;
   out->scratch_bytes = (int32_t)meta.scratch;
