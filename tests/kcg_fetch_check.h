@@ -76,6 +76,68 @@ int check_vm_schedule() {
   return 0;
 }
 
+// The counted waits for fragment reads (s_waitcnt lgkmcnt(n), n = StreamPlan::allowed(row)) against an explicit list of
+// the LDS read instructions in the order the K loop issues them: prologue (the B fragments of step 0, the first DA A
+// fragments, then a full wait); at the start of row i of a step the A fragment DA rows on (of this step, the next step or
+// the next tile's first step), behind the matrix instruction of slot slot_b(j) the B fragment j of the next step.  LDS
+// reads return in order: a wait with count n covers read X if at least n reads were issued after X.
+template <class P, class F>
+int check_lds_schedule() {
+  constexpr int ES = P::ES, TMI = P::WM / P::MF, TNI = P::WN / P::MF, DA = TMI - 1;
+  constexpr int RC = ES == 2 ? 2 : 4, NAI = P::AG ? 0 : (F::AK ? 1 : RC), NBI = RC;
+  typedef kcg::StreamPlan<TMI, TNI, DA, NAI, NBI> SP;
+  constexpr int KT = F::KT, KTT = F::KTT, SPW = P::SPW, SPWT = (F::KR + P::KS - 1) / P::KS;
+  static int last_read[2][64][2];                       // [operand][fragment][step parity] -> index of its last read instruction
+  int n = 0;                                            // read instructions issued so far
+  auto issue = [&](int is_b, int frag, int gstep, int count) {
+    n += count;
+    last_read[is_b][frag][gstep & 1] = n - 1;
+  };
+  auto bad = [](const char* what, int t, int s, int i, int have, int behind) {
+    printf("FAILED: lds schedule: %s (tile %d, step %d, row %d): waits with %d, %d reads were issued behind it\n", what, t, s, i, have, behind);
+    return 1;
+  };
+  for (int j = 0; j < TNI; ++j) issue(1, j, 0, NBI);
+  for (int i = 0; i < DA; ++i) issue(0, i, 0, NAI);
+  int complete = n;                                     // a full wait: everything issued so far has arrived
+  int gstep = 0;
+  for (int t = 0; t < KTT; ++t) {
+    const int ns = t < KT ? SPW : SPWT;
+    const bool h1 = t + 1 < KTT;
+    for (int s = 0; s < ns; ++s, ++gstep) {
+      const bool last = s == ns - 1, next = !last || h1;
+      for (int i = 0; i < TMI; ++i) {
+        // the wait at the start of the row
+        if (next) {
+          const int have = SP::allowed(i);
+          if (NAI > 0) {
+            const int x = last_read[0][i][gstep & 1];
+            if (x >= complete && n - 1 - x < have) return bad("A fragment", t, s, i, have, n - 1 - x);
+          }
+          if (i == 0)
+            for (int j = 0; j < TNI; ++j) {
+              const int x = last_read[1][j][gstep & 1];
+              if (x >= complete && n - 1 - x < have) return bad("B fragment", t, s, j, have, n - 1 - x);
+            }
+          if (n - have > complete) complete = n - have;
+        } else {
+          complete = n;
+        }
+        if (last && i == SP::RB) complete = n;           // the full wait in front of the barrier
+        // the A fragment DA rows on
+        if (NAI > 0) {
+          if (i + DA < TMI) issue(0, i + DA, gstep, NAI);
+          else if (!last || h1) issue(0, i + DA - TMI, gstep + 1, NAI);
+        }
+        for (int j = 0; j < TNI; ++j)
+          for (int jj = 0; jj < TNI; ++jj)
+            if (SP::slot_b(jj) == i * TNI + j && (!last || h1)) issue(1, jj, gstep + 1, NBI);
+      }
+    }
+  }
+  return 0;
+}
+
 int main() {
   typedef kcg::DirectPlan<Cfg> P;
   typedef kcg::FetchMap<Cfg> F;
@@ -86,6 +148,7 @@ int main() {
   if constexpr (P::AG) {
     if (check_vm_schedule<P, F>()) return 1;
   }
+  if (check_lds_schedule<P, F>()) return 1;
   constexpr int M = F::M, N = F::N, K = F::K, BM = F::BM, BN = F::BN, BK = F::BK, G = F::G, ES = F::ES, NW = F::NW;
   const long a_bytes = (long)M * K * ES, b_bytes = (long)K * N * ES;
   const int gy = (M + BM - 1) / BM, gx = (N + BN - 1) / BN;

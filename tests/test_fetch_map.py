@@ -5,7 +5,10 @@ written as host-callable code, so tests/kcg_fetch_check.h, appended to the `stru
 compiled for the host, can walk every block, K tile, wave, instruction and lane of a problem and check that no
 fetch leaves the operand buffers (the extents below put the ends of rows and of the buffers at every position
 inside a 16-byte chunk, with rows that start 2, 4, ... bytes off a 16-byte boundary) and that every element that
-exists lands where the fragment reads look for it.  No GPU needed: the parity tests on the GPU pin the rest."""
+exists lands where the fragment reads look for it.  The checker also lists the kernel's LDS read instructions in the
+order the K loop issues them and checks every counted wait (s_waitcnt lgkmcnt(n), n from StreamPlan::allowed) against that
+list: a fragment a row is about to use must have at least n reads issued behind it, or the wait would let the row start
+before the fragment has arrived.  No GPU needed: the parity tests on the GPU pin the rest."""
 import os
 import subprocess
 from concurrent.futures import ThreadPoolExecutor
