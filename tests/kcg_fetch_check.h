@@ -138,6 +138,48 @@ int check_lds_schedule() {
   return 0;
 }
 
+// The same for the global->LDS fetches of the ordinary build (both operands through LDS): at the barrier of tile t
+// the kernel waits with vmcnt(tiles_ahead(t) * NFETCH) for tile t+1 to have landed; every fetch of tile t+1 must have at
+// least that many fetches issued behind it (prologue: the first NST tiles, item by item; tile t: the items of tile t+NST
+// whose position is a slot of this tile, and those of tile t-1+NST whose position lies a period further on).
+template <class P, class F>
+int check_fetch_schedule() {
+  constexpr int SPW = P::SPW, TMI = P::WM / P::MF, TNI = P::WN / P::MF, NM = TMI * TNI, MT = SPW * NM;
+  constexpr int NST = P::NST, NFETCH = P::NFETCH, KTT = F::KTT;
+  constexpr int RB = 1, BAR = (SPW - 1) * NM + RB * TNI, SPREAD = NST >= 3 ? MT : MT - BAR;
+  static int last_of_tile[1 << 16];
+  if (KTT >= (1 << 16)) return 0;
+  int n = 0;
+  for (int t = 0; t < KTT; ++t) last_of_tile[t] = -1;
+  const int npro = NST < KTT ? NST : KTT;
+  for (int t = 0; t < npro; ++t) { n += NFETCH; last_of_tile[t] = n - 1; }
+  if (n - 1 - last_of_tile[0] < (npro - 1) * NFETCH && (npro - 1) * NFETCH <= 63) {
+    printf("FAILED: fetch schedule: the prologue's wait for tile 0 allows %d fetches in flight, %d were issued behind it\n", (npro - 1) * NFETCH, n - 1 - last_of_tile[0]);
+    return 1;
+  }
+  for (int t = 0; t < KTT; ++t) {
+    // slots in front of the barrier, the barrier's wait, then the rest (a partial last tile has fewer slots, but
+    // issues no fetches: nothing is left to fetch)
+    for (int q = 0; q < MT; ++q) {
+      if (q == BAR && t + 1 < KTT) {
+        const int newest = KTT - 1 < (t == 0 ? NST - 1 : t - 1 + NST) ? KTT - 1 : (t == 0 ? NST - 1 : t - 1 + NST);
+        const int ahead = newest - (t + 1) > 0 ? newest - (t + 1) : 0;
+        if (last_of_tile[t + 1] < 0 || n - 1 - last_of_tile[t + 1] < ahead * NFETCH) {
+          printf("FAILED: fetch schedule: the barrier of tile %d waits with %d, %d fetches were issued behind tile %d\n", t, ahead * NFETCH,
+                 last_of_tile[t + 1] < 0 ? -1 : n - 1 - last_of_tile[t + 1], t + 1);
+          return 1;
+        }
+      }
+      for (int f = 0; f < NFETCH; ++f) {
+        const int pos = BAR + (f * SPREAD) / NFETCH;
+        if (t + NST < KTT && pos == q) { ++n; last_of_tile[t + NST] = n - 1; }
+        if (t >= 1 && t - 1 + NST < KTT && SPREAD > MT - BAR && pos - MT == q) { ++n; last_of_tile[t - 1 + NST] = n - 1; }
+      }
+    }
+  }
+  return 0;
+}
+
 int main() {
   typedef kcg::DirectPlan<Cfg> P;
   typedef kcg::FetchMap<Cfg> F;
@@ -149,6 +191,9 @@ int main() {
     if (check_vm_schedule<P, F>()) return 1;
   }
   if (check_lds_schedule<P, F>()) return 1;
+  if constexpr (!P::AG) {
+    if (check_fetch_schedule<P, F>()) return 1;
+  }
   constexpr int M = F::M, N = F::N, K = F::K, BM = F::BM, BN = F::BN, BK = F::BK, G = F::G, ES = F::ES, NW = F::NW;
   const long a_bytes = (long)M * K * ES, b_bytes = (long)K * N * ES;
   const int gy = (M + BM - 1) / BM, gx = (N + BN - 1) / BN;
